@@ -46,8 +46,8 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
 }
 
 // Activations of a gated product, numbered as in the C interface: 0 = SiLU(g) * u; 1 = the clamped form
-// g' = min(g, limit), u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1).
-enum GateAct : int { kActSilu = 0, kActClampedSwish = 1, kGateActs = 2 };
+// g' = min(g, limit), u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1); 2 = max(g, 0) * u.
+enum GateAct : int { kActSilu = 0, kActClampedSwish = 1, kActRelu = 2, kGateActs = 3 };
 constexpr float kSwishSlope = 1.702f;
 __device__ __forceinline__ float gated_value(float g, float u, int act, float limit) {
   if (act == kActClampedSwish) {
@@ -55,6 +55,7 @@ __device__ __forceinline__ float gated_value(float g, float u, int act, float li
     u = fminf(fmaxf(u, -limit), limit);
     return g / (1.0f + expf(-kSwishSlope * g)) * (u + 1.0f);
   }
+  if (act == kActRelu) return fmaxf(g, 0.f) * u;
   return g / (1.0f + expf(-g)) * u;
 }
 

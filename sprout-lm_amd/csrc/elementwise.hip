@@ -155,14 +155,56 @@ __global__ void rope_cache_bf16_kernel(bf16_t* __restrict__ qkv, const int32_t* 
   }
 }
 
-// (cosine, sine) of positions[t] * inv_freq[d] for every token and pair: computed once per step for all layers.
-__global__ void rope_table_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq, int half,
+// (cosine, sine) of positions[t] * inv_freq[d] for every token and pair, both times `magnitude`: computed once per
+// step for all layers.  With inv_freq_tail (what the float32 table lost of the exact one) the angle, the sine and the
+// cosine are taken in float64.
+__global__ void rope_table_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  const float* __restrict__ inv_freq_tail, int half, float magnitude,
                                   float2* __restrict__ out, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   float sn, cs;
-  sincosf(float(positions[i / half]) * inv_freq[i % half], &sn, &cs);
+  if (inv_freq_tail) {
+    double sn64, cs64;
+    sincos(double(positions[i / half]) * (double(inv_freq[i % half]) + double(inv_freq_tail[i % half])), &sn64, &cs64);
+    sn = float(sn64 * double(magnitude));
+    cs = float(cs64 * double(magnitude));
+  } else {
+    sincosf(float(positions[i / half]) * inv_freq[i % half], &sn, &cs);
+    sn *= magnitude;
+    cs *= magnitude;
+  }
   out[i] = make_float2(cs, sn);
+}
+
+// x[i] *= factor
+__global__ void scale_kernel(float* __restrict__ x, float factor, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] *= factor;
+}
+
+// residual[t, c] += ma * sa[c] * a[t, c] (+ mb * sb[c] * b[t, c]): the sublayers' results, each times a learned vector
+// and a constant, join the residual stream in one pass.
+template <typename W>
+__global__ void scaled_add_kernel(float* __restrict__ residual, const float* __restrict__ a, const W* __restrict__ sa, float ma,
+                                  const float* __restrict__ b, const W* __restrict__ sb, float mb, int H, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int c = int(i % H);
+  float add = ma * (to_float(sa[c]) * a[i]);
+  if (b) add += mb * (to_float(sb[c]) * b[i]);
+  residual[i] += add;
+}
+
+// x[t, h, :] *= sigmoid(gate[t * gate_stride + h]): one number per token and head on that head's `width` numbers.
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ x, const T* __restrict__ gate, long long gate_stride, int heads, int width,
+                                 long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const long long th = i / width;
+  const float g = to_float(gate[(th / heads) * gate_stride + th % heads]);
+  x[i] = from_float<T>(to_float(x[i]) / (1.0f + expf(-g)));
 }
 
 template <typename T>
@@ -295,13 +337,49 @@ extern "C" int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, i
   return check_launch("sp_silu_mul");
 }
 
-extern "C" int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, int half, float* out, int T) {
+extern "C" int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, const float* inv_freq_tail, int half,
+                             float magnitude, float* out, int T) {
   SP_REQUIRE(T >= 0 && half > 0 && positions && inv_freq && out, "sp_rope_table: bad arguments");
   SP_REQUIRE(int64_t(T) * half < (int64_t(1) << 31), "sp_rope_table: too many entries");
   if (T == 0) return 0;
   const int n = T * half;
-  rope_table_kernel<<<(n + 255) / 256, 256, 0, (hipStream_t)stream>>>(positions, inv_freq, half, reinterpret_cast<float2*>(out), n);
+  rope_table_kernel<<<(n + 255) / 256, 256, 0, (hipStream_t)stream>>>(positions, inv_freq, inv_freq_tail, half, magnitude,
+                                                                      reinterpret_cast<float2*>(out), n);
   return check_launch("sp_rope_table");
+}
+
+extern "C" int sp_scale(void* stream, float* x, float factor, long long n) {
+  SP_REQUIRE(n >= 0 && (x || n == 0), "sp_scale: bad arguments");
+  if (n == 0) return 0;
+  scale_kernel<<<unsigned((n + 255) / 256), 256, 0, (hipStream_t)stream>>>(x, factor, n);
+  return check_launch("sp_scale");
+}
+
+extern "C" int sp_scaled_add(void* stream, float* residual, const float* a, int scale_dtype, const void* scale_a, float mult_a,
+                             const float* b, const void* scale_b, float mult_b, int T, int H) {
+  SP_REQUIRE(T >= 0 && H > 0 && residual && a && scale_a && (!b || scale_b), "sp_scaled_add: bad arguments");
+  SP_REQUIRE(scale_dtype == kF32 || scale_dtype == kBF16, "sp_scaled_add: unsupported dtype %d", scale_dtype);
+  if (T == 0) return 0;
+  const long long n = (long long)T * H;
+  const unsigned grid = unsigned((n + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (scale_dtype == kF32)
+    scaled_add_kernel<float><<<grid, 256, 0, s>>>(residual, a, (const float*)scale_a, mult_a, b, (const float*)scale_b, mult_b, H, n);
+  else
+    scaled_add_kernel<bf16_t><<<grid, 256, 0, s>>>(residual, a, (const bf16_t*)scale_a, mult_a, b, (const bf16_t*)scale_b, mult_b, H, n);
+  return check_launch("sp_scaled_add");
+}
+
+extern "C" int sp_head_gate(void* stream, int dtype, void* x, const void* gate, long long gate_stride, int T, int heads, int width) {
+  SP_REQUIRE(T >= 0 && heads > 0 && width > 0 && x && gate && gate_stride >= heads, "sp_head_gate: bad arguments");
+  SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_head_gate: unsupported dtype %d", dtype);
+  if (T == 0) return 0;
+  const long long n = (long long)T * heads * width;
+  const unsigned grid = unsigned((n + 255) / 256);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == kF32) head_gate_kernel<float><<<grid, 256, 0, s>>>((float*)x, (const float*)gate, gate_stride, heads, width, n);
+  else head_gate_kernel<bf16_t><<<grid, 256, 0, s>>>((bf16_t*)x, (const bf16_t*)gate, gate_stride, heads, width, n);
+  return check_launch("sp_head_gate");
 }
 
 extern "C" int sp_rope_cache(void* stream, int dtype, void* qkv, const int32_t* positions,

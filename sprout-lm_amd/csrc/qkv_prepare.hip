@@ -26,6 +26,8 @@ struct PrepareArgs {
   void* v_pool;                // [pages][nkv][width][page_size]
   int page_size;
   void* q_out;                 // [T, nq * width]
+  float magnitude;             // on every cosine and sine (1: a plain rotation)
+  int head_norm;               // every q and k head, after it has turned, is divided by its root mean square over dim (eps inside)
 };
 
 // Sum of the squares of n numbers over the whole block, as the scale of an RMS norm; every thread gets it.
@@ -37,9 +39,11 @@ __device__ __forceinline__ float row_scale(const T* __restrict__ x, int n, float
 }
 
 // One head of one token (query heads, then key heads, then value heads), by `count` threads of which this is `lane`.
+// `scratch` (16 floats): where `count` is the whole block, the head's sum of squares is taken over it; otherwise the
+// head belongs to one wave.
 template <typename T>
 __device__ __forceinline__ void prepare_head(const PrepareArgs& a, int t, int head, float q_scale, float k_scale, int slot,
-                                             int lane, int count) {
+                                             int lane, int count, float* scratch, bool whole_block) {
   const T* row = (const T*)a.proj + size_t(t) * a.stride;
   const int nq = a.nq, nkv = a.nkv, D = a.dim, V = a.vdim, W = a.width;
   const int page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
@@ -74,22 +78,34 @@ __device__ __forceinline__ void prepare_head(const PrepareArgs& a, int t, int he
     if (nw) x = to_float(from_float<T>((x * scale) * to_float(nw[e])));   // the storage type's rounding, as a norm kernel would leave it
     return x;
   };
+  // A turn by an angle times `magnitude` multiplies a pair's squares by magnitude^2, so the turned head's sum of squares
+  // needs no sines: the turned numbers' squares times magnitude^2, the others' as they are.
+  float unit = 1.f;
+  if (a.head_norm) {
+    float sq = 0.f;
+    const float m2 = a.magnitude * a.magnitude;
+    for (int d = lane; d < D; d += count) { const float x = normed(d); sq = fmaf(x * x, d < 2 * half ? m2 : 1.f, sq); }
+    sq = whole_block ? block_sum(sq, scratch) : wave_sum(sq);
+    unit = 1.0f / sqrtf(sq / float(D) + a.eps);
+  }
   for (int d = lane; d < W; d += count) {
     if (d >= D) { dst[d] = from_float<T>(0.f); continue; }
-    if (d >= 2 * half) { dst[d] = from_float<T>(normed(d)); continue; }
+    if (d >= 2 * half) { dst[d] = from_float<T>(normed(d) * unit); continue; }
     if (d >= half) continue;          // written by the owner of its pair
     float sn, cs;
     if (a.inv_freq_tail) {
       double sn64, cs64;
       sincos(double(a.positions[t]) * (double(a.inv_freq[d]) + double(a.inv_freq_tail[d])), &sn64, &cs64);
-      sn = float(sn64);
-      cs = float(cs64);
+      sn = float(sn64 * double(a.magnitude));
+      cs = float(cs64 * double(a.magnitude));
     } else {
       sincosf(float(a.positions[t]) * a.inv_freq[d], &sn, &cs);
+      sn *= a.magnitude;
+      cs *= a.magnitude;
     }
     const float x = normed(d), y = normed(d + half);
-    dst[d] = from_float<T>(x * cs - y * sn);
-    dst[d + half] = from_float<T>(y * cs + x * sn);
+    dst[d] = from_float<T>((x * cs - y * sn) * unit);
+    dst[d + half] = from_float<T>((y * cs + x * sn) * unit);
   }
 }
 
@@ -205,7 +221,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepareArgs a) {
       else scale = row_scale(whole, n, a.eps, scratch);
     }
     if constexpr (FOURS) prepare_head_fours(a, t, head, scale, scale, slot, threadIdx.x, blockDim.x);
-    else prepare_head<T>(a, t, head, scale, scale, slot, threadIdx.x, blockDim.x);
+    else prepare_head<T>(a, t, head, scale, scale, slot, threadIdx.x, blockDim.x, scratch, true);
     return;
   }
   float q_scale = 1.f, k_scale = 1.f;
@@ -221,7 +237,7 @@ __global__ __launch_bounds__(256) void qkv_prepare_kernel(PrepareArgs a) {
   const int wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
   for (int head = wave; head < heads; head += waves) {
     if constexpr (FOURS) prepare_head_fours(a, t, head, q_scale, k_scale, slot, threadIdx.x & 63, 64);
-    else prepare_head<T>(a, t, head, q_scale, k_scale, slot, threadIdx.x & 63, 64);
+    else prepare_head<T>(a, t, head, q_scale, k_scale, slot, threadIdx.x & 63, 64, scratch, false);
   }
 }
 
@@ -233,7 +249,7 @@ extern "C" int sp_qkv_prepare(void* stream, int dtype, const void* proj, long lo
                               int width, const void* q_norm, const void* k_norm, float eps, const int32_t* positions,
                               const float* inv_freq, const float* inv_freq_tail, int rotary_dim, const void* blend,
                               void* first, int keep_first, const int32_t* slot_mapping, void* k_pool, void* v_pool,
-                              int page_size, int num_pages, void* q_out, int T) {
+                              int page_size, int num_pages, void* q_out, int T, float magnitude, int head_norm) {
   SP_REQUIRE(T >= 0 && nq > 0 && nkv > 0 && dim > 0 && vdim > 0 && width >= dim && width >= vdim,
              "sp_qkv_prepare: bad sizes nq=%d nkv=%d dim=%d vdim=%d width=%d", nq, nkv, dim, vdim, width);
   SP_REQUIRE(stride >= (long long)(nq + nkv) * dim + (long long)nkv * vdim, "sp_qkv_prepare: a row of %lld numbers does not hold q, k and v", stride);
@@ -245,12 +261,12 @@ extern "C" int sp_qkv_prepare(void* stream, int dtype, const void* proj, long lo
   SP_REQUIRE(!slot_mapping || (k_pool && v_pool && page_size > 0 && num_pages > 0), "sp_qkv_prepare: bad cache geometry");
   if (T == 0) return 0;
   PrepareArgs a = {proj, stride, nq, nkv, dim, vdim, width, q_norm, k_norm, eps, positions, inv_freq, inv_freq_tail, rotary_dim,
-                   blend, first, keep_first, slot_mapping, k_pool, v_pool, page_size, q_out};
+                   blend, first, keep_first, slot_mapping, k_pool, v_pool, page_size, q_out, magnitude, head_norm};
   hipStream_t s = (hipStream_t)stream;
   SP_REQUIRE(nq + 2 * nkv <= 65535, "sp_qkv_prepare: %d heads are more than a launch's second dimension holds", nq + 2 * nkv);
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_qkv_prepare: unsupported dtype %d", dtype);
   auto eight = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7) == 0; };
-  const bool fours = dtype == kBF16 && !inv_freq_tail && dim % 4 == 0 && vdim % 4 == 0 && width % 4 == 0 && rotary_dim % 8 == 0 &&
+  const bool fours = dtype == kBF16 && !inv_freq_tail && !head_norm && magnitude == 1.0f && dim % 4 == 0 && vdim % 4 == 0 && width % 4 == 0 && rotary_dim % 8 == 0 &&
                      stride % 4 == 0 && eight(proj) && eight(q_out) && eight(q_norm) && eight(k_norm) && eight(first) &&
                      eight(k_pool);
   if (T * (nq + 2 * nkv) <= 2048) {      // few tokens: a block per head

@@ -5,7 +5,7 @@
 // implements is refused with an error, so another variant is an addition here and in the kernels, never a guess:
 //   pairing of a rotation     0 = halves of the rotated dimensions (d with d + rotary_dim / 2, "neox")
 //   activation of a gated product   0 = SiLU(g) * u (x / (1 + exp(-x)));  1 = clamped: g' = min(g, limit),
-//                                   u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1)
+//                                   u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1);  2 = max(g, 0) * u
 #pragma once
 #include <stdint.h>
 
@@ -53,7 +53,16 @@ int sp_qkv_rope_cache(void* stream, const void* x, const float* residual, int no
                       void* k_pool, void* v_pool, int T, int K, int nq, int nkv, int hd, int page_size,
                       const float* cos_sin, int pairing);
 // out [T][half][2] = (cosine, sine) of positions[t] * inv_freq[d]: the same for every layer of a step.
-int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, int half, float* out, int T);
+// Both times `magnitude`; with inv_freq_tail (what float32 lost of the exact table, may be null) angles in float64.
+int sp_rope_table(void* stream, const int32_t* positions, const float* inv_freq, const float* inv_freq_tail, int half,
+                  float magnitude, float* out, int T);
+// x[i] *= factor, float32
+int sp_scale(void* stream, float* x, float factor, long long n);
+// residual [T, H] += mult_a * scale_a[c] * a[t, c] (+ mult_b * scale_b[c] * b[t, c] where b is given); a, b float32.
+int sp_scaled_add(void* stream, float* residual, const float* a, int scale_dtype, const void* scale_a, float mult_a,
+                  const float* b, const void* scale_b, float mult_b, int T, int H);
+// x [T, heads, width] *= sigmoid(gate[t * gate_stride + head])
+int sp_head_gate(void* stream, int dtype, void* x, const void* gate, long long gate_stride, int T, int heads, int width);
 // out [T, I] = act(x . w[:I]^T, x . w[I:]^T) (times sigmoid(row_gate[t * row_gate_stride]) where row_gate, float32, is given)
 int sp_gate_up_silu(void* stream, const void* x, const float* residual, int norm_w_dtype, const void* norm_w, float eps,
                     const void* w, void* out, int T, int I, int K, int activation, float limit, const float* row_gate,
@@ -120,11 +129,13 @@ int sp_silu_mul(void* stream, int dtype, const void* gu, void* out, int T, int I
 // the root.  The first rotary_dim numbers of every q and k head turn (d with d + rotary_dim / 2) by positions *
 // inv_freq (+ inv_freq_tail: in float64).  blend (one number lambda of `dtype`): v <- (1 - lambda) v + lambda first[t];
 // keep_first: first[t] <- v instead.  q to q_out [T, nq * width]; k and v into the pools at slot_mapping (null or
-// negative: not cached), keys [pages][nkv][page][width], values [pages][nkv][width][page].
+// negative: not cached), keys [pages][nkv][page][width], values [pages][nkv][width][page].  Cosines and sines are
+// multiplied by `magnitude`; with head_norm every q and k head is divided, after it has turned, by its root mean
+// square over dim (eps inside the root, no weight).
 int sp_qkv_prepare(void* stream, int dtype, const void* proj, long long stride, int nq, int nkv, int dim, int vdim, int width,
                    const void* q_norm, const void* k_norm, float eps, const int32_t* positions, const float* inv_freq,
                    const float* inv_freq_tail, int rotary_dim, const void* blend, void* first, int keep_first,
-                   const int32_t* slot_mapping, void* k_pool, void* v_pool, int page_size, int num_pages, void* q_out, int T);
+                   const int32_t* slot_mapping, void* k_pool, void* v_pool, int page_size, int num_pages, void* q_out, int T, float magnitude, int head_norm);
 
 // dst (dst_dtype) = src (src_dtype), n elements
 
@@ -251,4 +262,26 @@ int sp_route_combine_identity(void* stream, const float* y, const int32_t* row_o
 // `iterations` x 4 independent 32x32x16 bfloat16 products a wave; *flops receives the operations of one launch).
 int sp_probe_read(void* stream, const void* data, int64_t bytes, int blocks, float* sink);
 int sp_probe_mfma(void* stream, int blocks, int iterations, float* sink, double* flops);
+// A gated linear recurrence over `width` channels behind a causal convolution of `taps` taps per channel.
+// proj [T, stride] holds two branches of `width` numbers (biases added): at y_off the gate branch before its activation,
+// at x_off the convolution's input.  u = conv(x) (conv_w [width, taps], last column the current token's; inputs before a
+// request's first token are zeros); the channels fall into `blocks` equal parts, part b's gates are
+// r = sigmoid(wa[b] u_b + ba[b]), i = sigmoid(wi[b] u_b + bi[b]) with the matrices INPUT-major ([blocks, in, out]);
+// a = exp(-8 r softplus(lam)), S <- a S + sqrt(1 - a^2) i u per token, out [T, width] = S * gelu_tanh(y).
+// state [slots, width] and tail [slots, taps - 1, width] (the last inputs of the convolution, oldest first; null for one
+// tap) are float32 rows indexed by state_slots[request]; decay and drive are float32 scratch [T, width].
+int sp_rglru_takes(int width, int blocks, int taps);
+int sp_rglru(void* stream, int dtype, const void* proj, long long stride, int y_off, int x_off, int width, int blocks, int taps,
+             const void* conv_w, const void* conv_b, const void* wa, const void* ba, const void* wi, const void* bi,
+             const void* lam, const int32_t* q_start, const int32_t* q_len, const int32_t* seq_of_token,
+             const int32_t* state_slots, float* state, float* tail, float* decay, float* drive, void* out, int T, int n_seqs);
+
+// Retention: per head S <- decay[h] S + k v^T, o = S^T q, with q and k turned by the angles of cos_sin ([T, rotary_dim / 2, 2]
+// of sp_rope_table: the first rotary_dim numbers of a head, d with d + rotary_dim / 2) and k times dim^(-1/2); o is divided
+// by its root mean square over vdim (eps inside the root) and multiplied by silu(gate).  proj [T, stride] holds q, k
+// (heads * dim), v and the gate (heads * vdim) at their offsets; state float32 [slots, heads, dim, vdim]; out [T, heads * vdim].
+int sp_retention_takes(int dim, int vdim);
+int sp_retention(void* stream, int dtype, const void* proj, long long stride, int q_off, int k_off, int v_off, int g_off, int heads,
+                 int dim, int vdim, int rotary_dim, const float* cos_sin, const float* decay, float eps, const int32_t* q_start,
+                 const int32_t* q_len, const int32_t* state_slots, float* state, void* out, int T, int n_seqs);
 }

@@ -99,7 +99,7 @@ def main(argv=None) -> int:
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at a time (each rounded up to 64)")
     parser.add_argument("--block-size", type=int, default=PAGE_TOKENS, help="tokens per cache page (divides 64)")
-    parser.add_argument("--max-sequences", type=int, default=16)
+    parser.add_argument("--max-sequences", type=int, default=4, help="requests that are live at a time (state slots)")
     args = parser.parse_args(argv)
     if args.max_tokens <= 0 or args.block_size <= 0 or 64 % args.block_size:
         parser.error("--max-tokens must be positive and --block-size must divide 64")

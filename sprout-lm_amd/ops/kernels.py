@@ -64,7 +64,8 @@ def _ptr(t):
 ROTARY_PAIRINGS = {"halves": 0}          # dimension d turns with d + rotary_dim / 2 ("neox"); the latent mixer's own
                                          # kernel (latent_prepare) turns neighbours (2i, 2i + 1)
 GATE_ACTIVATIONS = {"silu": 0,           # silu(g) * u
-                    "clamped_swish": 1}  # g' = min(g, limit), u' = clamp(u, -limit, limit): g' * sigmoid(1.702 g') * (u' + 1)
+                    "clamped_swish": 1,  # g' = min(g, limit), u' = clamp(u, -limit, limit): g' * sigmoid(1.702 g') * (u' + 1)
+                    "relu": 2}           # max(g, 0) * u
 SCORE_STAGES = {"scaled_dot": 0,         # what stands between q . k and the softmax: the scale and nothing else,
                 "capped": 1}             # or the scaled product s squashed to cap * tanh(s / cap)
 MAX_HEAD_DIM = 512                       # the largest head size any attention kernel takes
@@ -357,11 +358,13 @@ def route_combine_identity(y: torch.Tensor, row_of_pair, ids: torch.Tensor, weig
 
 def qkv_prepare(proj: torch.Tensor, nq: int, nkv: int, dim: int, vdim: int, width: int, q_out: torch.Tensor, positions=None,
                 inv_freq=None, inv_freq_tail=None, rotary_dim: int = 0, q_norm=None, k_norm=None, eps: float = 0.0,
-                blend=None, first=None, keep_first: bool = False, slot_mapping=None, k_pool=None, v_pool=None) -> None:
+                blend=None, first=None, keep_first: bool = False, slot_mapping=None, k_pool=None, v_pool=None,
+                magnitude: float = 1.0, head_norm: bool = False) -> None:
     """From rows of projections [q | k | v] (heads of `dim`, `dim` and `vdim` numbers): optional RMS norm over the whole
     q row and the whole k row, optional rotation of the heads' first rotary_dim numbers, optional blend of the values
     with `first` (or `first` <- values), q to q_out [T, nq * width], k and v into pools that keep both `width` wide
-    (zeros behind); see sprout_hip.h."""
+    (zeros behind); cosines and sines times `magnitude`; with `head_norm` every q and k head is divided, after turning,
+    by its root mean square over dim (`eps` inside the root); see sprout_hip.h."""
     _gpu(proj, "projections"); _gpu(q_out, "queries")
     T, stride = proj.shape
     if stride < (nq + nkv) * dim + nkv * vdim or tuple(q_out.shape) != (T, nq * width) or q_out.dtype != proj.dtype:
@@ -393,7 +396,8 @@ def qkv_prepare(proj: torch.Tensor, nq: int, nkv: int, dim: int, vdim: int, widt
                                    _ptr(inv_freq) if rotary_dim else None, _ptr(inv_freq_tail) if rotary_dim else None,
                                    int(rotary_dim), _ptr(blend), _ptr(first), int(bool(keep_first)), _ptr(slot_mapping),
                                    _ptr(k_pool) if slot_mapping is not None else None,
-                                   _ptr(v_pool) if slot_mapping is not None else None, page_size, num_pages, q_out.data_ptr(), T))
+                                   _ptr(v_pool) if slot_mapping is not None else None, page_size, num_pages, q_out.data_ptr(), T,
+                                   float(magnitude), int(bool(head_norm))))
 
 
 STORE, ACCUMULATE, STORE_F32 = 0, 1, 2
@@ -705,14 +709,124 @@ def qkv_rope_cache(w: torch.Tensor, bias, q_out: torch.Tensor, positions, inv_fr
                                       variant_code(ROTARY_PAIRINGS, pairing, "rotation pairing")))
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor) -> None:
-    """out[t, d] = (cos, sin) of positions[t] * inv_freq[d]; out float32 [T, len(inv_freq), 2]."""
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out: torch.Tensor, inv_freq_tail=None,
+               magnitude: float = 1.0) -> None:
+    """out[t, d] = magnitude * (cos, sin) of positions[t] * inv_freq[d]; out float32 [T, len(inv_freq), 2].  With
+    `inv_freq_tail` (what the float32 table lost of the exact one) angles, sines and cosines are taken in float64."""
     _gpu(inv_freq, "inv_freq"); _gpu(out, "rotation table")
     T, half = out.shape[0], inv_freq.numel()
     _ints(positions, T, "positions")
     if inv_freq.dtype != torch.float32 or out.dtype != torch.float32 or tuple(out.shape) != (T, half, 2):
         raise KernelError("rope_table: inv_freq float32 [half] and out float32 [T, half, 2] expected")
-    check(library().sp_rope_table(_stream(), positions.data_ptr(), inv_freq.data_ptr(), half, out.data_ptr(), T))
+    if inv_freq_tail is not None:
+        _gpu(inv_freq_tail, "inv_freq_tail")
+        if inv_freq_tail.dtype != torch.float32 or inv_freq_tail.numel() != half:
+            raise KernelError("rope_table: inv_freq_tail must be float32 and as long as inv_freq")
+    check(library().sp_rope_table(_stream(), positions.data_ptr(), inv_freq.data_ptr(), _ptr(inv_freq_tail), half,
+                                  float(magnitude), out.data_ptr(), T))
+
+
+def scale(x: torch.Tensor, factor: float) -> None:
+    """x *= factor, float32, in place."""
+    _gpu(x, "scaled tensor")
+    if x.dtype != torch.float32:
+        raise KernelError("scale: float32 expected")
+    check(library().sp_scale(_stream(), x.data_ptr(), float(factor), x.numel()))
+
+
+def scaled_add(residual: torch.Tensor, a: torch.Tensor, scale_a: torch.Tensor, mult_a: float, b=None, scale_b=None,
+               mult_b: float = 0.0) -> None:
+    """residual [T, H] += mult_a * scale_a * a (+ mult_b * scale_b * b): float32 rows times learned vectors of H numbers."""
+    _gpu(residual, "residual"); _gpu(a, "first summand"); _gpu(scale_a, "first scale")
+    T, H = residual.shape
+    if residual.dtype != torch.float32 or a.dtype != torch.float32 or a.shape[0] < T or a.shape[1] != H or scale_a.numel() != H:
+        raise KernelError(f"scaled_add: residual {tuple(residual.shape)} {residual.dtype}, summand {tuple(a.shape)} {a.dtype}, "
+                          f"scale of {scale_a.numel()} do not fit")
+    if b is not None:
+        _gpu(b, "second summand"); _gpu(scale_b, "second scale")
+        if b.dtype != torch.float32 or b.shape[0] < T or b.shape[1] != H or scale_b.numel() != H or scale_b.dtype != scale_a.dtype:
+            raise KernelError("scaled_add: the second summand does not fit the first")
+    check(library().sp_scaled_add(_stream(), residual.data_ptr(), a.data_ptr(), _code(scale_a, "scale"), scale_a.data_ptr(),
+                                  float(mult_a), _ptr(b), _ptr(scale_b) if b is not None else None, float(mult_b), T, H))
+
+
+def head_gate(x: torch.Tensor, gate: torch.Tensor, gate_offset: int, heads: int, width: int) -> None:
+    """x [T, heads * width] *= sigmoid(gate[t, gate_offset + head]), in place; x and gate of one dtype."""
+    _gpu(x, "gated heads"); _gpu(gate, "head gate")
+    T = x.shape[0]
+    if x.shape[1] != heads * width or gate.dtype != x.dtype or gate.shape[0] < T or gate_offset < 0 or gate_offset + heads > gate.shape[1]:
+        raise KernelError(f"head_gate: heads {tuple(x.shape)} {x.dtype} and gate {tuple(gate.shape)} {gate.dtype} do not fit")
+    check(library().sp_head_gate(_stream(), _code(x, "gated heads"), x.data_ptr(), gate.data_ptr() + gate_offset * gate.element_size(),
+                                 gate.shape[1], T, heads, width))
+
+
+def rglru_takes(width: int, blocks: int, taps: int) -> bool:
+    return bool(library().sp_rglru_takes(int(width), int(blocks), int(taps)))
+
+
+def rglru(proj: torch.Tensor, y_off: int, x_off: int, width: int, blocks: int, taps: int, conv_w, conv_b, wa, ba, wi, bi, lam,
+          q_start, q_len, seq_of_token, state_slots, n_seqs: int, state: torch.Tensor, tail, decay: torch.Tensor,
+          drive: torch.Tensor, out: torch.Tensor) -> None:
+    """The gated linear recurrence of sp_rglru (sprout_hip.h) on a step's tokens.  `wa`, `wi`: [blocks, in, out]."""
+    T, n = out.shape[0], width // max(blocks, 1)
+    for t, what in ((proj, "projections"), (out, "recurrence output"), (state, "recurrent state"), (decay, "decay scratch"),
+                    (drive, "drive scratch")):
+        _gpu(t, what)
+    if proj.shape[0] < T or out.dtype != proj.dtype or tuple(out.shape) != (T, width) or max(y_off, x_off) + width > proj.shape[1]:
+        raise KernelError(f"rglru: projections {tuple(proj.shape)} {proj.dtype} and output {tuple(out.shape)} {out.dtype} do not fit")
+    for t, shape, what in ((conv_w, (width, taps), "conv"), (conv_b, (width,), "conv bias"), (wa, (blocks, n, n), "gate matrices"),
+                           (wi, (blocks, n, n), "gate matrices"), (ba, (blocks, n), "gate bias"), (bi, (blocks, n), "gate bias"),
+                           (lam, (width,), "lam")):
+        _gpu(t, what)
+        if tuple(t.shape) != shape or t.dtype != proj.dtype:
+            raise KernelError(f"rglru: {what} must be {shape} {proj.dtype}, got {tuple(t.shape)} {t.dtype}")
+    for t, count, what in ((q_start, n_seqs, "q_start"), (q_len, n_seqs, "q_len"), (state_slots, n_seqs, "state_slots"),
+                           (seq_of_token, T, "seq_of_token")):
+        _ints(t, count, what)
+    if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != width:
+        raise KernelError("rglru: the state must be float32 [slots, width]")
+    if taps > 1:
+        _gpu(tail, "convolution tail")
+        if tail.dtype != torch.float32 or tuple(tail.shape) != (state.shape[0], taps - 1, width):
+            raise KernelError("rglru: the convolution's kept inputs must be float32 [slots, taps - 1, width]")
+    for t in (decay, drive):
+        if t.dtype != torch.float32 or t.numel() < T * width:
+            raise KernelError("rglru: scratch must hold float32 [T, width]")
+    check(library().sp_rglru(_stream(), _code(proj, "projections"), proj.data_ptr(), proj.shape[1], y_off, x_off, width, blocks,
+                             taps, conv_w.data_ptr(), conv_b.data_ptr(), wa.data_ptr(), ba.data_ptr(), wi.data_ptr(), bi.data_ptr(),
+                             lam.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), seq_of_token.data_ptr(), state_slots.data_ptr(),
+                             state.data_ptr(), _ptr(tail) if taps > 1 else None, decay.data_ptr(), drive.data_ptr(),
+                             out.data_ptr(), T, n_seqs))
+
+
+def retention_takes(dim: int, vdim: int) -> bool:
+    return bool(library().sp_retention_takes(int(dim), int(vdim)))
+
+
+def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, heads: int, dim: int, vdim: int,
+              rotary_dim: int, cos_sin, decay: torch.Tensor, eps: float, q_start, q_len, state_slots, n_seqs: int,
+              state: torch.Tensor, out: torch.Tensor) -> None:
+    """Retention of sp_retention (sprout_hip.h) on a step's tokens; `cos_sin`: rope_table of the step's positions."""
+    T = out.shape[0]
+    _gpu(proj, "projections"); _gpu(out, "retention output"); _gpu(state, "retention state"); _gpu(decay, "decays")
+    if proj.shape[0] < T or out.dtype != proj.dtype or tuple(out.shape) != (T, heads * vdim):
+        raise KernelError(f"retention: projections {tuple(proj.shape)} {proj.dtype} and output {tuple(out.shape)} {out.dtype} do not fit")
+    if max(q_off, k_off) + heads * dim > proj.shape[1] or max(v_off, g_off) + heads * vdim > proj.shape[1] or min(q_off, k_off, v_off, g_off) < 0:
+        raise KernelError("retention: a row of projections does not hold q, k, v and the gate")
+    if decay.dtype != torch.float32 or decay.numel() != heads:
+        raise KernelError(f"retention: decays must be {heads} float32 values")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, dim, vdim):
+        raise KernelError(f"retention: the state must be float32 [slots, {heads}, {dim}, {vdim}]")
+    if rotary_dim:
+        _gpu(cos_sin, "rotation table")
+        if cos_sin.dtype != torch.float32 or cos_sin.shape[0] < T or tuple(cos_sin.shape[1:]) != (rotary_dim // 2, 2):
+            raise KernelError("retention: the rotation table must be float32 [T, rotary_dim / 2, 2]")
+    for t, what in ((q_start, "q_start"), (q_len, "q_len"), (state_slots, "state_slots")):
+        _ints(t, n_seqs, what)
+    check(library().sp_retention(_stream(), _code(proj, "projections"), proj.data_ptr(), proj.shape[1], q_off, k_off, v_off, g_off,
+                                 heads, dim, vdim, rotary_dim, _ptr(cos_sin) if rotary_dim else None, decay.data_ptr(), float(eps),
+                                 q_start.data_ptr(), q_len.data_ptr(), state_slots.data_ptr(), state.data_ptr(), out.data_ptr(),
+                                 T, n_seqs))
 
 
 def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm_weight=None, eps: float = 0.0,

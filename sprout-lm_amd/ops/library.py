@@ -38,7 +38,15 @@ def _declare(lib):
                            c_int, c_int],
         "sp_qkv_rope_cache": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_int, c_void, c_void, c_void,
                               c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_int],
-        "sp_rope_table": [c_void, c_void, c_void, c_int, c_void, c_int],
+        "sp_rope_table": [c_void, c_void, c_void, c_void, c_int, c_float, c_void, c_int],
+        "sp_scale": [c_void, c_void, c_float, c_i64],
+        "sp_scaled_add": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_float, c_int, c_int],
+        "sp_head_gate": [c_void, c_int, c_void, c_void, c_i64, c_int, c_int, c_int],
+        "sp_rglru_takes": [c_int] * 3,
+        "sp_rglru": [c_void, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_int] + [c_void] * 16 + [c_int, c_int],
+        "sp_retention_takes": [c_int] * 2,
+        "sp_retention": [c_void, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_void,
+                         c_float, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int, c_float, c_void, c_i64],
         "sp_gate_up_silu_f32_takes": [c_int, c_int, c_int],
         "sp_gate_up_silu_f32": [c_void, c_void, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int, c_float, c_void, c_i64],
@@ -68,7 +76,8 @@ def _declare(lib):
                             c_int, c_void, c_void, c_void, c_void],
         "sp_route_combine_identity": [c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_void, c_int, c_void, c_int, c_int],
         "sp_qkv_prepare": [c_void, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_int, c_void, c_void, c_float, c_void,
-                           c_void, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_void, c_int],
+                           c_void, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_int, c_void, c_int,
+                           c_float, c_int],
         "sp_expert_down": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_void, c_int, c_int, c_int, c_int],
         "sp_route_combine": [c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_int],
         "sp_probe_read": [c_void, c_void, c_i64, c_int, c_void],

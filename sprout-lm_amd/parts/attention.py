@@ -42,6 +42,9 @@ class Attention(Mixer):
         if (scores == "capped") != (softcap is not None and softcap > 0):
             raise ConfigError(f"Capped scores need a positive cap, and a cap the score stage 'capped'; got {scores!r}, {softcap!r}.")
         self.scores, self.softcap = scores, float(softcap or 0.0)
+        if getattr(position, "magnitude", 1.0) != 1.0:
+            raise ConfigError("This mixer's kernels turn by plain cosines and sines; a position encoding that scales them needs "
+                              "the mixer 'sink_attention'.")
         if head_dim % 2 and getattr(position, "rotary_dim", 0):
             raise ConfigError(f"A rotation needs an even head size, got {head_dim}.")
         self.hidden, self.heads, self.kv_heads, self.head_dim = hidden, heads, kv_heads, head_dim

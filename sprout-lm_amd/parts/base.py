@@ -12,7 +12,7 @@ from typing import Callable
 from ..weights.loader import TensorSpec
 
 _REGISTRIES: dict[str, dict[str, type]] = {
-    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "embedding": {}, "head": {},
+    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "embedding": {}, "head": {}, "scale": {},
 }
 
 
@@ -148,6 +148,14 @@ class FeedForward(Part):
     def forward_from_residual(self, ctx, norm, residual) -> bool:
         """Optional shortcut, as Mixer.forward_from_residual."""
         return False
+
+
+class BranchScale(Part):
+    """What multiplies a sublayer's result on its way into the residual stream: a learned vector, a constant, both."""
+
+    def add(self, ctx, residual, branch, other=None, other_branch=None):
+        """residual += scale(branch) (+ other's scale(other_branch)); the branches are float32 [T, hidden]."""
+        raise NotImplementedError
 
 
 class Block(Part):

@@ -68,3 +68,39 @@ class ParallelBlock(Block):
         self.mixer.forward(ctx, h, residual, caches.get("mixer"))
         if self.ffn is not None:
             self.ffn.forward(ctx, h2, residual)
+
+
+@register_part("block", "parallel_scaled")
+class ScaledParallelBlock(Block):
+    """x += scale_a(mixer(norm(x))) + scale_b(feed_forward(norm(x))): ONE norm whose output both sublayers read, and each
+    sublayer's result goes through a part of its own (a learned vector, a constant) before the sum.  The sublayers add
+    into float32 rows of their own, which are cleared first; `ffn` (and its scale) may be absent."""
+
+    graph_safe = True
+
+    graph_safe_portions = True
+
+    def __init__(self, mixer_norm, mixer, mixer_scale, ffn=None, ffn_scale=None):
+        self.mixer_norm, self.mixer, self.mixer_scale, self.ffn, self.ffn_scale = mixer_norm, mixer, mixer_scale, ffn, ffn_scale
+
+    def parts(self):
+        named = {"mixer_norm": self.mixer_norm, "mixer": self.mixer, "mixer_scale": self.mixer_scale}
+        if self.ffn is not None:
+            named.update({"ffn": self.ffn, "ffn_scale": self.ffn_scale})
+        return named
+
+    def forward(self, ctx, residual, caches):
+        import torch
+        T, H = residual.shape
+        h = ctx.buffer("normed", (T, H), ctx.act_dtype)
+        self.mixer_norm.forward(ctx, residual, h)
+        both = ctx.buffer("branches", (2, T, H), torch.float32)
+        if self.ffn is None:
+            both[0].zero_()
+            self.mixer.forward(ctx, h, both[0], caches.get("mixer"))
+            self.mixer_scale.add(ctx, residual, both[0])
+            return
+        both.zero_()
+        self.mixer.forward(ctx, h, both[0], caches.get("mixer"))
+        self.ffn.forward(ctx, h, both[1])
+        self.mixer_scale.add(ctx, residual, both[0], self.ffn_scale, both[1])

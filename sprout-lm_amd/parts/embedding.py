@@ -62,14 +62,14 @@ class BigramEmbedding(Part):
 
 @register_part("head", "linear_head")
 class LinearHead(Part):
-    """logits = W . x in float32.  With `tied`, W is the embedding table and the head has no tensor."""
+    """logits = (W . x) * scale in float32.  With `tied`, W is the embedding table and the head has no tensor."""
 
     graph_safe = True
 
     graph_safe_portions = True
 
-    def __init__(self, vocab: int, hidden: int, tied: bool, tensor: str = "weight"):
-        self.vocab, self.hidden, self.tied, self.tensor = vocab, hidden, tied, tensor
+    def __init__(self, vocab: int, hidden: int, tied: bool, tensor: str = "weight", scale: float = 1.0):
+        self.vocab, self.hidden, self.tied, self.tensor, self.scale = vocab, hidden, tied, tensor, float(scale)
         self.table = None
 
     def tensors(self):
@@ -85,6 +85,8 @@ class LinearHead(Part):
 
     def forward(self, ctx, h, logits):
         ops.gemm(h, self.table, logits)
+        if self.scale != 1.0:
+            ops.scale(logits, self.scale)
 
     def weight_elements(self) -> int:
         return self.vocab * self.hidden      # the output matrix is read whole, also where it is the embedding table

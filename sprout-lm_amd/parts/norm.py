@@ -8,24 +8,25 @@ from .base import Norm, NormFold, register_part
 
 @register_part("norm", "rmsnorm")
 class RMSNorm(Norm):
-    """y = x / sqrt(mean(x^2) + eps) * weight; sums in float32, the weight is used as it is."""
+    """y = x / sqrt(mean(x^2) + eps) * weight; sums in float32, the weight is used as it is.  `tensor`: the local
+    name of the weight."""
 
     graph_safe = True
 
     graph_safe_portions = True
 
-    def __init__(self, size: int, eps: float):
-        self.size, self.eps = size, eps
+    def __init__(self, size: int, eps: float, tensor: str = "weight"):
+        self.size, self.eps, self.tensor = size, eps, tensor
 
     def tensors(self):
-        return {"weight": TensorSpec((self.size,), "vector", "one_plus_normal")}
+        return {self.tensor: TensorSpec((self.size,), "vector", "one_plus_normal")}
 
     def forward(self, ctx, x, out, rows=None):
-        ops.rmsnorm(x, self.w["weight"], self.eps, out, rows)
+        ops.rmsnorm(x, self.w[self.tensor], self.eps, out, rows)
         return out
 
     def fold(self):
-        return NormFold("rms", self.w["weight"], self.eps)
+        return NormFold("rms", self.w[self.tensor], self.eps)
 
 
 @register_part("norm", "layernorm")

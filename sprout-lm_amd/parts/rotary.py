@@ -10,6 +10,12 @@ from .base import PositionEncoding, register_part
 class NeoxRotary(PositionEncoding):
     """Pair (d, d + rotary_dim/2) of a head turns by position * theta^(-2d / rotary_dim).
 
+    `scaling` (None, or factor / original / fast / slow): frequencies are blended between f_d and f_d / factor along a
+    ramp over the pair index d, and cosine and sine are multiplied by `magnitude` = 0.1 ln(factor) + 1 ("YaRN"): with
+    turns(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(turns(fast)), 0), hi =
+    min(ceil(turns(slow)), rotary_dim - 1) and ramp_d = clamp((d - lo) / max(hi - lo, 0.001), 0, 1) pair d turns by
+    position * (f_d / factor * ramp_d + f_d * (1 - ramp_d)).
+
     The table of inverse frequencies is computed in float64 and kept in float32; angles, sines
     and cosines are float32 in the kernel.  For float32 models the part also keeps what the float32
     table lost (`inv_freq_tail`), and the kernel computes angle, sine and cosine in float64: a float32
@@ -22,17 +28,34 @@ class NeoxRotary(PositionEncoding):
     graph_safe_portions = True
     pairing = "halves"      # which dimensions turn together, as the kernels name it (ops.ROTARY_PAIRINGS)
 
-    def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None):
+    def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None, scaling: dict | None = None):
+        import math
         self.head_dim, self.theta = head_dim, theta
         self.rotary_dim = head_dim if rotary_dim is None else rotary_dim
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= head_dim:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {head_dim}.")
+        self.scaling = dict(scaling) if scaling else None
+        self.magnitude = 0.1 * math.log(float(self.scaling["factor"])) + 1.0 if self.scaling else 1.0
         self.inv_freq = None
         self.inv_freq_tail = None
 
+    def frequencies(self) -> torch.Tensor:
+        """The exact (float64) frequency of every pair."""
+        import math
+        n = self.rotary_dim
+        d = torch.arange(n // 2, dtype=torch.float64)
+        freq = float(self.theta) ** (-2.0 * d / n)
+        if not self.scaling:
+            return freq
+        factor, original = float(self.scaling["factor"]), float(self.scaling["original"])
+        turns = lambda t: n * math.log(original / (2.0 * math.pi * t)) / (2.0 * math.log(float(self.theta)))
+        lo = max(math.floor(turns(float(self.scaling["fast"]))), 0)
+        hi = min(math.ceil(turns(float(self.scaling["slow"]))), n - 1)
+        ramp = ((d - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        return freq / factor * ramp + freq * (1.0 - ramp)
+
     def prepare(self, device, dtype):
-        d = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64)
-        exact = float(self.theta) ** (-d / self.rotary_dim)
+        exact = self.frequencies()
         self.inv_freq = exact.to(torch.float32).to(device)
         if dtype == torch.float32:
             self.inv_freq_tail = (exact - exact.to(torch.float32).to(torch.float64)).to(torch.float32).to(device)
@@ -41,12 +64,13 @@ class NeoxRotary(PositionEncoding):
         """(cosine, sine) of every token's angles, float32 [T, rotary_dim / 2, 2]: the same in every layer, so
         the first layer of a step that asks computes it and the others find it in the step's context."""
         from .. import ops
-        key = ("rotary_neox", self.rotary_dim, float(self.theta))
+        scaling = tuple(sorted(self.scaling.items())) if self.scaling else ()
+        key = ("rotary_neox", self.rotary_dim, float(self.theta), scaling)
         found = ctx.shared.get(key)
         if found is None:
-            found = ctx.buffer(f"rotation_table_{self.rotary_dim}_{float(self.theta)!r}",
-                               (ctx.n_tokens, self.rotary_dim // 2, 2), torch.float32)
-            ops.rope_table(ctx.positions, self.inv_freq, found)
+            name = f"rotation_table_{self.rotary_dim}_{float(self.theta)!r}" + (f"_{hash(scaling) & 0xffffffff:x}" if scaling else "")
+            found = ctx.buffer(name, (ctx.n_tokens, self.rotary_dim // 2, 2), torch.float32)
+            ops.rope_table(ctx.positions, self.inv_freq, found, inv_freq_tail=self.inv_freq_tail, magnitude=self.magnitude)
             ctx.shared[key] = found
         return found
 

@@ -36,6 +36,11 @@ class SinkAttention(Mixer):
     softmax's denominator also holds exp(sink_h), a tensor of one number per head that has no key and no value.
     value_mix: None, "first" (this layer's values are kept for the step under `value_key`) or "blend" (v <- (1 - l) v +
     l first, l the one-number tensor `blend`); the blended values are what is cached.  W_o mixes the heads' outputs.
+    head_norm: after turning, every q and k head is divided by its root mean square over dim (`eps` inside the root, no
+    weight).  sink_value: a constant logit in the denominator in place of learned ones (0.0: the denominator holds one
+    more 1).  head_gate: head h's output is multiplied by sigmoid((W_g h)_h), W_g a tensor [heads, hidden] whose rows ride
+    behind those of q, k and v in the one product (the last name of `tensors`).  A position encoding may scale its
+    cosines and sines (`magnitude`).
 
     Keys (dim numbers) and values (vdim numbers) lie in the cache at one common width (`padded_width`), zeros behind, so
     the attention kernels see equal head sizes; W_o gets columns of zeros to match.  What a step does: one product for
@@ -51,8 +56,9 @@ class SinkAttention(Mixer):
     def __init__(self, hidden: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, position, qkv_bias: bool = False,
                  qk_norm: bool = False, eps: float = 0.0, softcap: float | None = None, mask_chunk: int | None = None,
                  window: int | None = None, sinks: bool = True, value_mix: str | None = None, value_key: str = "first_values",
-                 page_tokens: int | None = None,
-                 tensors: tuple = ("q", "k", "v", "o", ".b", ".norm", "vmix", "sink")):
+                 page_tokens: int | None = None, head_norm: bool = False, sink_value: float | None = None,
+                 head_gate: bool = False,
+                 tensors: tuple = ("q", "k", "v", "o", ".b", ".norm", "vmix", "sink", "g")):
         if min(hidden, heads, kv_heads, dim, vdim) <= 0 or heads % kv_heads:
             raise ConfigError(f"Attention needs positive sizes and heads in whole groups, got heads={heads} kv_heads={kv_heads} "
                               f"dim={dim} vdim={vdim}.")
@@ -63,6 +69,10 @@ class SinkAttention(Mixer):
         for name, n in (("mask_chunk", mask_chunk), ("window", window)):
             if n is not None and n <= 0:
                 raise ConfigError(f"{name} must be positive, got {n!r}.")
+        if sinks and sink_value is not None:
+            raise ConfigError("The denominator's extra term is learned (sinks) or a constant (sink_value), not both.")
+        if qkv_bias and head_gate:
+            raise ConfigError("A gate per head rides in the q/k/v product, which then carries no biases.")
         rotary = getattr(position, "rotary_dim", 0)
         if rotary and (getattr(position, "pairing", None) != "halves" or rotary > dim or rotary % 2):
             raise ConfigError(f"This mixer turns the first {rotary} numbers of a head of {dim} in halves; the position "
@@ -76,7 +86,8 @@ class SinkAttention(Mixer):
         self.scale, self.position, self.qkv_bias, self.qk_norm, self.eps = float(scale), position, qkv_bias, qk_norm, float(eps)
         self.softcap, self.mask_chunk, self.window, self.sinks = softcap, mask_chunk, window, sinks
         self.value_mix, self.value_key, self.page_tokens = value_mix, value_key, page_tokens
-        self.names = tuple(tensors)
+        self.head_norm, self.sink_value, self.head_gate = bool(head_norm), sink_value, bool(head_gate)
+        self.names = tuple(tensors) + ("g",) * (9 - len(tensors))
 
     # ------------------------------------------------------------------ what it keeps and costs
     def _reach(self):
@@ -92,11 +103,12 @@ class SinkAttention(Mixer):
 
     def flops(self, tokens: int, pairs: int = 0) -> float:
         q, k, v = self.heads * self.dim, self.kv_heads * self.dim, self.kv_heads * self.vdim
-        projections = 2.0 * tokens * self.hidden * (q + k + v) + 2.0 * tokens * self.heads * self.vdim * self.hidden
+        projections = 2.0 * tokens * self.hidden * (q + k + v + (self.heads if self.head_gate else 0)) \
+            + 2.0 * tokens * self.heads * self.vdim * self.hidden
         return projections + 2.0 * self.heads * (self.dim + self.vdim) * pairs
 
     def tensors(self):
-        q, k, v, o, b, norm, blend, sink = self.names
+        q, k, v, o, b, norm, blend, sink, gate = self.names
         H, G, D, V = self.heads, self.kv_heads, self.dim, self.vdim
         out = {q: TensorSpec((H * D, self.hidden)), k: TensorSpec((G * D, self.hidden)), v: TensorSpec((G * V, self.hidden)),
                o: TensorSpec((self.hidden, H * V))}
@@ -110,16 +122,21 @@ class SinkAttention(Mixer):
             out[blend] = TensorSpec((), "vector")
         if self.sinks:
             out[sink] = TensorSpec((H,), "vector")
+        if self.head_gate:
+            out[gate] = TensorSpec((H, self.hidden))
         return out
 
     def bind(self, tensors):
-        q, k, v, o, b, norm, blend, sink = self.names
-        self.w_qkv = torch.cat([tensors[q], tensors[k], tensors[v]], dim=0).contiguous()
+        q, k, v, o, b, norm, blend, sink, gate = self.names
+        self.w_qkv = torch.cat([tensors[q], tensors[k], tensors[v]] + ([tensors[gate]] if self.head_gate else []), dim=0).contiguous()
+        self.gate_offset = (self.heads + self.kv_heads) * self.dim + self.kv_heads * self.vdim
         self.b_qkv = torch.cat([tensors[q + b], tensors[k + b], tensors[v + b]], dim=0).contiguous() if self.qkv_bias else None
         self.w_q_norm = tensors[q + norm] if self.qk_norm else None
         self.w_k_norm = tensors[k + norm] if self.qk_norm else None
         self.blend = tensors[blend].reshape(1).contiguous() if self.value_mix == "blend" else None
         self.sink = tensors[sink].to(torch.float32).contiguous() if self.sinks else None
+        if self.sink_value is not None:
+            self.sink = torch.full((self.heads,), float(self.sink_value), dtype=torch.float32, device=self.w_qkv.device)
         w_o = tensors[o]
         if self.width != self.vdim:      # columns of zeros where the cached values are wider than the values
             wide = torch.zeros(self.hidden, self.heads, self.width, dtype=w_o.dtype, device=w_o.device)
@@ -156,12 +173,15 @@ class SinkAttention(Mixer):
                         inv_freq_tail=getattr(self.position, "inv_freq_tail", None) if rotary and proj.dtype == torch.float32 else None,
                         rotary_dim=rotary, q_norm=self.w_q_norm, k_norm=self.w_k_norm, eps=self.eps, blend=self.blend,
                         first=first, keep_first=self.value_mix == "first", slot_mapping=cache.slot_mapping if writes else None,
-                        k_pool=cache.k if writes else None, v_pool=cache.v if writes else None)
+                        k_pool=cache.k if writes else None, v_pool=cache.v if writes else None,
+                        magnitude=getattr(self.position, "magnitude", 1.0) if rotary else 1.0, head_norm=self.head_norm)
         mixed = ctx.buffer("attn", (T, H * W), ctx.act_dtype)
-        project = (self.w_o, residual)
+        project = None if self.head_gate else (self.w_o, residual)    # a gate stands between the heads' outputs and W_o
         if ops.attention(queries, H * W, cache.k, cache.v, cache.block_tables, ctx.attention, mixed, H, G, W, self.window,
                          self.scale, workspace=lambda n: ctx.buffer("attention_partials", (n,), torch.float32),
                          kind=ctx.attention_kind, project=project, scores="capped" if self.softcap else "scaled_dot",
                          softcap=self.softcap or 0.0, sinks=self.sink, mask_chunk=self.mask_chunk):
             return
+        if self.head_gate:
+            ops.head_gate(mixed, proj, self.gate_offset, H, W)
         ops.gemm(mixed, self.w_o, residual, accumulate=True)

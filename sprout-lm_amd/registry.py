@@ -68,6 +68,9 @@ def _register_builtin():
     from .config.bogilix import BogilixConfig
     from .models.bogilix import build_bogilix
     register_architecture(BogilixConfig.architecture, BogilixConfig, build_bogilix)
+    from .config.morarax import MoraraxConfig
+    from .models.morarax import build_morarax
+    register_architecture(MoraraxConfig.architecture, MoraraxConfig, build_morarax)
 
 
 _register_builtin()
