@@ -564,10 +564,11 @@ def test_variants_without_a_kernel_are_refused_by_the_library_itself():
     assert lib.sp_fused_supported(ops.FUSED_ROPE, 8, 1152, 896, 64, 64, 0, 0) == 1
     assert lib.sp_fused_supported(ops.FUSED_ROPE, 8, 1152, 896, 64, 64, 0, 1) == 0
     assert lib.sp_fused_supported(ops.FUSED_SILU, 8, 9728, 896, 0, 0, 0, 1) == 1
-    assert lib.sp_fused_supported(ops.FUSED_SILU, 8, 9728, 896, 0, 0, 0, 2) == 0
+    assert lib.sp_fused_supported(ops.FUSED_SILU, 8, 9728, 896, 0, 0, 0, 2) == 1
+    assert lib.sp_fused_supported(ops.FUSED_SILU, 8, 9728, 896, 0, 0, 0, 3) == 0
     assert not ops.fused_supported(ops.FUSED_SILU, 8, 9728, 896, variant="gelu")
-    with pytest.raises(ops.KernelError, match="activation 'relu'"):
-        ops.silu_mul(gu, out, activation="relu")
+    with pytest.raises(ops.KernelError, match="activation 'gelu'"):
+        ops.silu_mul(gu, out, activation="gelu")
     # what stands between q . k and the softmax is such a parameter of the attention entry points
     q = torch.zeros(1, 32, device=DEV)
     kp, vp = torch.zeros(2, 1, 8, 16, device=DEV), torch.zeros(2, 1, 16, 8, device=DEV)
