@@ -19,7 +19,7 @@ part of a step that the host spends planning and launching, which the look-ahead
 another prompt is prefilled 256 tokens a step; with --pressure SHARE, the batch in a pool too small for its
 requests at the headline sizes.
 
-    python bench.py --design megozen|bogilix [--sizes s,m,l] [--design-batches 1,8,64]
+    python bench.py --design megozen|bogilix|morarax [--sizes s,m,l] [--design-batches 1,8,64]
 
 times the Megozen presets instead (latent attention, routed experts), each beside the dense model of equal width,
 layers, vocabulary and work per token, and prints a line of its own; the default workload above is untouched.
@@ -314,7 +314,7 @@ def design_points(design: str, sizes: list[str], dtype: str, dtype_name: str, ba
 
 def main() -> int:
     parser = argparse.ArgumentParser()
-    parser.add_argument("--design", default=None, choices=["megozen", "bogilix"],
+    parser.add_argument("--design", default=None, choices=["megozen", "bogilix", "morarax"],
                         help="time nothing but this design's presets (--sizes) beside dense models of equal size: "
                              "decode at --design-batches and --context, prefill of --prefill-tokens; prints a line of its own")
     parser.add_argument("--sizes", default="s,m,l", help="with --design: which of its presets")

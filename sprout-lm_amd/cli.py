@@ -2,7 +2,7 @@
 
     python -m sprout_lm_amd demo [--json] [--pressure]
     python -m sprout_lm_amd generate MODEL_DIR --prompt-ids 1,2,3 [--max-new-tokens N] ...
-    python -m sprout_lm_amd init --preset tiny-a|tiny-b|qwen2.5-0.5b|megozen-s|bogilix-s|... | --config FILE  --out DIR [--seed N]
+    python -m sprout_lm_amd init --preset tiny-a|tiny-b|qwen2.5-0.5b|megozen-s|bogilix-s|morarax-s|... | --config FILE  --out DIR [--seed N]
 
 `demo` is the counterpart of the reference's src/demo.ts, with the reference's two options: a few requests on a
 tiny random model, told round by round (--json: the same as one JSON document; --pressure: a pool so small that
@@ -112,6 +112,35 @@ PRESETS.update({
     # large: 8 layers of width 4,096, 32 heads of 128 over 4 key/value heads
     "bogilix-l": _bogilix_preset(4096, 8, 32, 4, 128, 128, 2048, 62, 2, 6, 1024, 2048, 8192, 32768),
     "bogilix-l-dense": _dense_twin(4096, 8, 32, 4, 8192, 32768),
+})
+
+
+def _morarax_preset(width: int, layers: int, heads: int, kv_heads: int, dim: int, state_heads: int, blocks: int, ff: int,
+                    vocab: int) -> dict:
+    """A Morarax configuration: layers in the order retention, gated recurrence, retention, attention, again and again.
+    Attention heads of `dim` with blended frequencies; retention heads of 64 keys beside 128 values with decays
+    1 - 2^(-5 - 4 h / heads); a recurrence as wide as the model in `blocks` parts behind four taps."""
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                 "rot": {"base": 500000.0, "dims": dim // 2, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    retention = {"heads": state_heads, "dim": 64, "vdim": 128, "rot": {"base": 10000.0, "dims": 64},
+                 "decay": [1.0 - 2.0 ** (-5.0 - 4.0 * h / state_heads) for h in range(state_heads)]}
+    recurrence = {"width": width, "blocks": blocks, "conv": 4}
+    order = (("retention", retention), ("rglru", recurrence), ("retention", retention), ("attention", attention))
+    entries = [{"type": order[i % 4][0], "mixer": order[i % 4][1], "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]
+    return {"architecture": "Morarax", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "logit_scale": 0.25, "layers": entries}
+
+
+PRESETS.update({
+    # small: 8 layers of width 1,024; attention of 16 heads of 64 over 2 key/value heads, retention of 8 heads
+    "morarax-s": _morarax_preset(1024, 8, 16, 2, 64, 8, 16, 2048, 32768),
+    "morarax-s-dense": _dense_twin(1024, 8, 16, 2, 2048, 32768),
+    # medium: 12 layers of width 2,048; attention of 16 heads of 128, retention of 16 heads
+    "morarax-m": _morarax_preset(2048, 12, 16, 2, 128, 16, 16, 4224, 32768),
+    "morarax-m-dense": _dense_twin(2048, 12, 16, 2, 4224, 32768),
+    # large: 8 layers of width 4,096; attention of 32 heads of 128 over 4 key/value heads, retention of 32 heads
+    "morarax-l": _morarax_preset(4096, 8, 32, 4, 128, 32, 16, 8192, 32768),
+    "morarax-l-dense": _dense_twin(4096, 8, 32, 4, 8192, 32768),
 })
 
 

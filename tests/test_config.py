@@ -93,7 +93,7 @@ def test_sizes_that_no_kernel_takes_are_refused_when_the_parts_are_built():
         PartPlan("feed_forward", "gated_mlp", {"hidden": 8, "inner": 8, "activation": "gelu"}).make()
     with pytest.raises(ops.KernelError, match="rotation pairing 'interleaved'"):
         ops.kernels.variant_code(ops.ROTARY_PAIRINGS, "interleaved", "rotation pairing")
-    assert ops.ROTARY_PAIRINGS == {"halves": 0} and ops.GATE_ACTIVATIONS == {"silu": 0, "clamped_swish": 1}
+    assert ops.ROTARY_PAIRINGS == {"halves": 0} and ops.GATE_ACTIVATIONS == {"silu": 0, "clamped_swish": 1, "relu": 2}
     with pytest.raises(ValueError, match="needs a positive limit"):
         PartPlan("feed_forward", "gated_mlp", {"hidden": 8, "inner": 8, "activation": "clamped_swish"}).make()
     with pytest.raises(ConfigError, match="score stage 'soft_cap'"):
