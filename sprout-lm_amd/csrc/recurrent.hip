@@ -132,6 +132,97 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(LruArgs a) {
   }
 }
 
+// The same walk for long portions, in three passes over chunks of kScanChunk tokens so that a request's tokens are shared
+// out over the chip: every chunk's own product of decays and its sum from zero; per channel the few chunks one after the
+// other, which leaves every chunk the state it starts from (and the request its new state and convolution inputs); then
+// every chunk again from that state, writing the output.  carry_a, carry_b: float32 [requests * chunks, width].
+constexpr int kScanChunk = 64;
+
+__global__ __launch_bounds__(256) void rglru_chunk_local_kernel(LruArgs a, float* __restrict__ carry_a,
+                                                                float* __restrict__ carry_b, int chunks) {
+  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= a.width) return;
+  const int first = a.q_start[s] + ci * kScanChunk, end = min(first + kScanChunk, a.q_start[s] + a.q_len[s]);
+  if (first >= end) return;
+  float A = 1.f, B = 0.f;
+  int t = first;
+  for (; t + 8 <= end; t += 8) {
+    float d[8], g[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      d[j] = a.decay[size_t(t + j) * a.width + c];
+      g[j] = a.drive[size_t(t + j) * a.width + c];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      B = fmaf(d[j], B, g[j]);
+      A *= d[j];
+    }
+  }
+  for (; t < end; ++t) {
+    const float d = a.decay[size_t(t) * a.width + c];
+    B = fmaf(d, B, a.drive[size_t(t) * a.width + c]);
+    A *= d;
+  }
+  carry_a[size_t(blockIdx.x) * a.width + c] = A;
+  carry_b[size_t(blockIdx.x) * a.width + c] = B;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_chunk_carry_kernel(LruArgs a, const float* __restrict__ carry_a,
+                                                                float* __restrict__ carry_b, int chunks) {
+  const int s = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= a.width) return;
+  const int start = a.q_start[s], n = a.q_len[s], slot = a.state_slots[s];
+  const int used = (n + kScanChunk - 1) / kScanChunk;
+  float S = a.state[size_t(slot) * a.width + c];
+  for (int ci = 0; ci < used; ++ci) {
+    const size_t at = (size_t(s) * chunks + ci) * a.width + c;
+    const float A = carry_a[at], B = carry_b[at];
+    carry_b[at] = S;          // what the chunk starts from
+    S = fmaf(A, S, B);
+  }
+  a.state[size_t(slot) * a.width + c] = S;
+  const T* proj = (const T*)a.proj;
+  const int keep = a.taps - 1;
+  float* tail = a.tail + size_t(slot) * keep * a.width;
+  for (int p = 0; p < keep; ++p) {
+    const int j = n - keep + p;
+    tail[size_t(p) * a.width + c] = j >= 0 ? to_float(proj[size_t(start + j) * a.stride + a.x_off + c])
+                                           : tail[size_t(p + n) * a.width + c];
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_chunk_apply_kernel(LruArgs a, const float* __restrict__ carry_b, int chunks) {
+  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= a.width) return;
+  const int first = a.q_start[s] + ci * kScanChunk, end = min(first + kScanChunk, a.q_start[s] + a.q_len[s]);
+  if (first >= end) return;
+  const T* proj = (const T*)a.proj;
+  T* out = (T*)a.out;
+  float S = carry_b[size_t(blockIdx.x) * a.width + c];
+  int t = first;
+  for (; t + 8 <= end; t += 8) {
+    float d[8], g[8], y[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      d[j] = a.decay[size_t(t + j) * a.width + c];
+      g[j] = a.drive[size_t(t + j) * a.width + c];
+      y[j] = to_float(proj[size_t(t + j) * a.stride + a.y_off + c]);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      S = fmaf(d[j], S, g[j]);
+      out[size_t(t + j) * a.width + c] = from_float<T>(S * gelu_tanh(y[j]));
+    }
+  }
+  for (; t < end; ++t) {
+    S = fmaf(a.decay[size_t(t) * a.width + c], S, a.drive[size_t(t) * a.width + c]);
+    out[size_t(t) * a.width + c] = from_float<T>(S * gelu_tanh(to_float(proj[size_t(t) * a.stride + a.y_off + c])));
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ retention
 struct RetentionArgs {
   const void* proj;            // [T, stride]: q and k (heads * dim each), v and the gate (heads * vdim each) at their offsets
@@ -224,6 +315,257 @@ __global__ __launch_bounds__(256) void retention_kernel(RetentionArgs a) {
   }
 }
 
+// The same sums for long portions, chunk by chunk, in three passes so that a request's tokens are shared out over the chip.
+// With a chunk's tokens 0 .. n-1, its state before them S0 and decay g:
+//   o_i = g^(i+1) S0^T q_i + sum_(j<=i) g^(i-j) (q_i . k_j) v_j        S_n = g^n S0 + sum_j g^(n-1-j) k_j v_j^T
+// Only powers of g with exponents >= 0 appear (nothing is divided by a power), so a small decay loses nothing.
+// First every chunk's own sum U = sum_j g^(n-1-j) k_j v_j^T; then per state element the chunks one after the other, which
+// leaves in U's place the state each chunk starts from; then every chunk's outputs.  scratch: float32
+// [requests * chunks, heads, dim, vdim].  A thread block is 8 rows of 32 threads.
+template <typename T>
+__device__ __forceinline__ float turned(const T* src, const float* cos_sin, size_t t, int d, int half) {
+  if (d < 2 * half) {
+    const int p = d < half ? d : d - half;
+    const float2 cs = reinterpret_cast<const float2*>(cos_sin)[t * half + p];
+    const float x = to_float(src[p]), y = to_float(src[p + half]);
+    return d < half ? x * cs.x - y * cs.y : y * cs.x + x * cs.y;
+  }
+  return to_float(src[d]);
+}
+
+template <typename T, int CV>
+__global__ __launch_bounds__(256) void retention_chunk_local_kernel(RetentionArgs a, float* __restrict__ scratch, int chunks, int C) {
+  extern __shared__ float lds[];      // k [C][D + 1] (times its power of the decay), v [C][V]
+  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, h = blockIdx.y;
+  const int D = a.dim, V = a.vdim, half = a.rotary_dim / 2, DP = D + 1;
+  const int first = a.q_start[s] + ci * C, len = min(C, a.q_start[s] + a.q_len[s] - first);
+  if (len <= 0) return;
+  float* ks = lds;
+  float* vs = lds + C * DP;
+  const float gamma = a.decay[h], k_scale = 1.0f / sqrtf(float(D));
+  const T* proj = (const T*)a.proj;
+  for (int e = threadIdx.x; e < len * D; e += blockDim.x) {
+    const int j = e / D, d = e % D;
+    const T* src = proj + size_t(first + j) * a.stride + a.k_off + h * D;
+    ks[j * DP + d] = (turned(src, a.cos_sin, size_t(first + j), d, half) * k_scale) * powf(gamma, float(len - 1 - j));
+  }
+  for (int e = threadIdx.x; e < len * V; e += blockDim.x) {
+    const int j = e / V, v = e % V;
+    vs[e] = to_float(proj[size_t(first + j) * a.stride + a.v_off + h * V + v]);
+  }
+  __syncthreads();
+  const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;
+  float* U = scratch + (size_t(blockIdx.x) * a.heads + h) * D * V;
+  for (int d0 = 0; d0 < D; d0 += 32) {
+    float acc[4][CV];
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int c = 0; c < CV; ++c) acc[r][c] = 0.f;
+    for (int j = 0; j < len; ++j) {
+      float kk[4], vv[CV];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int d = d0 + ty + 8 * r;
+        kk[r] = d < D ? ks[j * DP + d] : 0.f;
+      }
+#pragma unroll
+      for (int c = 0; c < CV; ++c) {
+        const int v = tx + 32 * c;
+        vv[c] = v < V ? vs[j * V + v] : 0.f;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < CV; ++c) acc[r][c] = fmaf(kk[r], vv[c], acc[r][c]);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int d = d0 + ty + 8 * r;
+#pragma unroll
+      for (int c = 0; c < CV; ++c) {
+        const int v = tx + 32 * c;
+        if (d < D && v < V) U[size_t(d) * V + v] = acc[r][c];
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void retention_chunk_carry_kernel(RetentionArgs a, float* __restrict__ scratch, int chunks, int C) {
+  const int s = blockIdx.x, h = blockIdx.y, DV = a.dim * a.vdim, e = blockIdx.z * blockDim.x + threadIdx.x;
+  if (e >= DV) return;
+  const int n = a.q_len[s], slot = a.state_slots[s], used = (n + C - 1) / C;
+  const float gamma = a.decay[h];
+  float* kept = a.state + (size_t(slot) * a.heads + h) * DV + e;
+  float S = *kept;
+  for (int ci = 0; ci < used; ++ci) {
+    float* at = scratch + ((size_t(s) * chunks + ci) * a.heads + h) * DV + e;
+    const float U = *at;
+    *at = S;          // what the chunk starts from
+    S = fmaf(powf(gamma, float(min(C, n - ci * C))), S, U);
+  }
+  *kept = S;
+}
+
+template <typename T, int C, int CV>
+__global__ __launch_bounds__(256) void retention_chunk_apply_kernel(RetentionArgs a, const float* __restrict__ scratch, int chunks) {
+  extern __shared__ float lds[];      // q, k [C][D + 1], v [C][V], weights [C][C + 1], powers of the decay [C + 1]
+  constexpr int RPT = C / 8, JC = (C + 31) / 32, CP = C + 1;
+  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, h = blockIdx.y;
+  const int D = a.dim, V = a.vdim, half = a.rotary_dim / 2, DP = D + 1;
+  const int first = a.q_start[s] + ci * C, len = min(C, a.q_start[s] + a.q_len[s] - first);
+  if (len <= 0) return;
+  float* qs = lds;
+  float* ks = qs + C * DP;
+  float* vs = ks + C * DP;
+  float* ps = vs + C * V;
+  float* pw = ps + C * CP;
+  const float gamma = a.decay[h], k_scale = 1.0f / sqrtf(float(D));
+  const T* proj = (const T*)a.proj;
+  T* out = (T*)a.out;
+  for (int e = threadIdx.x; e < 2 * C * D; e += blockDim.x) {
+    const bool is_k = e >= C * D;
+    const int r = is_k ? e - C * D : e, j = r / D, d = r % D;
+    float value = 0.f;
+    if (j < len) {
+      const T* src = proj + size_t(first + j) * a.stride + (is_k ? a.k_off : a.q_off) + h * D;
+      value = turned(src, a.cos_sin, size_t(first + j), d, half);
+      if (is_k) value *= k_scale;
+    }
+    (is_k ? ks : qs)[j * DP + d] = value;
+  }
+  for (int e = threadIdx.x; e < C * V; e += blockDim.x) {
+    const int j = e / V, v = e % V;
+    vs[e] = j < len ? to_float(proj[size_t(first + j) * a.stride + a.v_off + h * V + v]) : 0.f;
+  }
+  for (int e = threadIdx.x; e <= C; e += blockDim.x) pw[e] = powf(gamma, float(e));
+  __syncthreads();
+  const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;
+  {
+    float acc[RPT][JC];
+#pragma unroll
+    for (int r = 0; r < RPT; ++r)
+#pragma unroll
+      for (int c = 0; c < JC; ++c) acc[r][c] = 0.f;
+    for (int d = 0; d < D; ++d) {
+      float qq[RPT], kk[JC];
+#pragma unroll
+      for (int r = 0; r < RPT; ++r) qq[r] = qs[(ty + 8 * r) * DP + d];
+#pragma unroll
+      for (int c = 0; c < JC; ++c) {
+        const int j = tx + 32 * c;
+        kk[c] = j < C ? ks[j * DP + d] : 0.f;
+      }
+#pragma unroll
+      for (int r = 0; r < RPT; ++r)
+#pragma unroll
+        for (int c = 0; c < JC; ++c) acc[r][c] = fmaf(qq[r], kk[c], acc[r][c]);
+    }
+#pragma unroll
+    for (int r = 0; r < RPT; ++r)
+#pragma unroll
+      for (int c = 0; c < JC; ++c) {
+        const int i = ty + 8 * r, j = tx + 32 * c;
+        if (j < C) ps[i * CP + j] = j <= i ? acc[r][c] * pw[i - j] : 0.f;
+      }
+  }
+  __syncthreads();
+  float o[RPT][CV];
+#pragma unroll
+  for (int r = 0; r < RPT; ++r)
+#pragma unroll
+    for (int c = 0; c < CV; ++c) o[r][c] = 0.f;
+  const float* S0 = scratch + (size_t(blockIdx.x) * a.heads + h) * D * V;
+  for (int d = 0; d < D; ++d) {      // what the tokens before the chunk left
+    float qq[RPT], ss[CV];
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) qq[r] = qs[(ty + 8 * r) * DP + d];
+#pragma unroll
+    for (int c = 0; c < CV; ++c) {
+      const int v = tx + 32 * c;
+      ss[c] = v < V ? S0[size_t(d) * V + v] : 0.f;
+    }
+#pragma unroll
+    for (int r = 0; r < RPT; ++r)
+#pragma unroll
+      for (int c = 0; c < CV; ++c) o[r][c] = fmaf(qq[r], ss[c], o[r][c]);
+  }
+#pragma unroll
+  for (int r = 0; r < RPT; ++r)
+#pragma unroll
+    for (int c = 0; c < CV; ++c) o[r][c] *= pw[ty + 8 * r + 1];
+  for (int j = 0; j < len; ++j) {      // the chunk's own tokens
+    float pp[RPT], vv[CV];
+#pragma unroll
+    for (int r = 0; r < RPT; ++r) pp[r] = ps[(ty + 8 * r) * CP + j];
+#pragma unroll
+    for (int c = 0; c < CV; ++c) {
+      const int v = tx + 32 * c;
+      vv[c] = v < V ? vs[j * V + v] : 0.f;
+    }
+#pragma unroll
+    for (int r = 0; r < RPT; ++r)
+#pragma unroll
+      for (int c = 0; c < CV; ++c) o[r][c] = fmaf(pp[r], vv[c], o[r][c]);
+  }
+#pragma unroll
+  for (int r = 0; r < RPT; ++r) {
+    const int i = ty + 8 * r;
+    float squares = 0.f;
+#pragma unroll
+    for (int c = 0; c < CV; ++c) squares = fmaf(o[r][c], o[r][c], squares);      // columns past V hold zeros
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) squares += __shfl_xor(squares, off);
+    if (i >= len) continue;
+    const float unit = 1.0f / sqrtf(squares / float(V) + a.eps);
+    const T* row = proj + size_t(first + i) * a.stride;
+#pragma unroll
+    for (int c = 0; c < CV; ++c) {
+      const int v = tx + 32 * c;
+      if (v < V) {
+        const float g = to_float(row[a.g_off + h * V + v]);
+        out[(size_t(first + i) * a.heads + h) * V + v] = from_float<T>((o[r][c] * unit) * (g * sigmoid(g)));
+      }
+    }
+  }
+}
+
+constexpr int kRetentionLongPortion = 8;      // a step whose longest portion has more tokens takes the chunks
+
+static size_t retention_chunk_lds(int C, int dim, int vdim) {
+  return sizeof(float) * (size_t(2) * C * (dim + 1) + size_t(C) * vdim + size_t(C) * (C + 1) + C + 1);
+}
+// Tokens per chunk: the most whose tiles fit 64 KB of LDS (0: none do).
+static int retention_chunk_tokens(int dim, int vdim) {
+  for (int C : {64, 32, 16})
+    if (retention_chunk_lds(C, dim, vdim) <= 64 * 1024) return C;
+  return 0;
+}
+
+template <typename T, int CV>
+static int launch_retention_chunks(hipStream_t s, const RetentionArgs& a, int n_seqs, int max_q_len, float* scratch) {
+  const int C = retention_chunk_tokens(a.dim, a.vdim), chunks = (max_q_len + C - 1) / C, DV = a.dim * a.vdim;
+  SP_REQUIRE((long long)n_seqs * chunks < (1 << 30), "sp_retention: too many chunks");
+  const dim3 grid(n_seqs * chunks, a.heads);
+  const size_t local_lds = sizeof(float) * (size_t(C) * (a.dim + 1) + size_t(C) * a.vdim);
+  retention_chunk_local_kernel<T, CV><<<grid, 256, local_lds, s>>>(a, scratch, chunks, C);
+  retention_chunk_carry_kernel<<<dim3(n_seqs, a.heads, (DV + 255) / 256), 256, 0, s>>>(a, scratch, chunks, C);
+  const size_t lds = retention_chunk_lds(C, a.dim, a.vdim);
+  if (C == 64) retention_chunk_apply_kernel<T, 64, CV><<<grid, 256, lds, s>>>(a, scratch, chunks);
+  else if (C == 32) retention_chunk_apply_kernel<T, 32, CV><<<grid, 256, lds, s>>>(a, scratch, chunks);
+  else retention_chunk_apply_kernel<T, 16, CV><<<grid, 256, lds, s>>>(a, scratch, chunks);
+  return check_launch("sp_retention (chunks)");
+}
+
+template <typename T>
+static int launch_retention_chunks(hipStream_t s, const RetentionArgs& a, int n_seqs, int max_q_len, float* scratch) {
+  const int cv = (a.vdim + 31) / 32;
+  if (cv <= 1) return launch_retention_chunks<T, 1>(s, a, n_seqs, max_q_len, scratch);
+  if (cv <= 2) return launch_retention_chunks<T, 2>(s, a, n_seqs, max_q_len, scratch);
+  if (cv <= 4) return launch_retention_chunks<T, 4>(s, a, n_seqs, max_q_len, scratch);
+  return launch_retention_chunks<T, 8>(s, a, n_seqs, max_q_len, scratch);
+}
+
 template <typename T>
 static int launch_retention(hipStream_t s, const RetentionArgs& a, int n_seqs, int rows, int threads, size_t lds) {
   const dim3 grid(n_seqs, a.heads);
@@ -238,6 +580,13 @@ static int launch_retention(hipStream_t s, const RetentionArgs& a, int n_seqs, i
 
 using namespace sprout;
 
+// float32 numbers of the scratch that a step whose longest portion has max_q_len tokens needs for its scan in chunks
+// (0: the scan walks each request in one go and needs none).
+extern "C" long long sp_rglru_carry_floats(int width, int n_seqs, int max_q_len) {
+  if (max_q_len <= 2 * kScanChunk) return 0;
+  return 2LL * n_seqs * ((max_q_len + kScanChunk - 1) / kScanChunk) * width;
+}
+
 extern "C" int sp_rglru_takes(int width, int blocks, int taps) {
   return width > 0 && blocks > 0 && width % blocks == 0 && taps >= 1 && taps <= 64 && width / blocks <= 2048;
 }
@@ -246,7 +595,7 @@ extern "C" int sp_rglru(void* stream, int dtype, const void* proj, long long str
                         int taps, const void* conv_w, const void* conv_b, const void* wa, const void* ba, const void* wi,
                         const void* bi, const void* lam, const int32_t* q_start, const int32_t* q_len,
                         const int32_t* seq_of_token, const int32_t* state_slots, float* state, float* tail, float* decay,
-                        float* drive, void* out, int T, int n_seqs) {
+                        float* drive, void* out, int T, int n_seqs, int max_q_len, float* carry) {
   SP_REQUIRE(sp_rglru_takes(width, blocks, taps), "sp_rglru: no kernel for width=%d blocks=%d taps=%d", width, blocks, taps);
   SP_REQUIRE(T >= 0 && n_seqs >= 0 && y_off >= 0 && x_off >= 0 && stride >= y_off + width && stride >= x_off + width,
              "sp_rglru: rows of %lld numbers do not hold both branches", stride);
@@ -274,6 +623,22 @@ extern "C" int sp_rglru(void* stream, int dtype, const void* proj, long long str
   if (check_launch("sp_rglru (gates)")) return 1;
   const int scan_threads = width >= 256 ? 256 : (width + 63) / 64 * 64;
   const dim3 scan_grid(n_seqs, (width + scan_threads - 1) / scan_threads);
+  if (carry && max_q_len > 2 * kScanChunk) {      // a long portion: its chunks side by side
+    const int chunks = (max_q_len + kScanChunk - 1) / kScanChunk;
+    SP_REQUIRE((long long)n_seqs * chunks < (1 << 30), "sp_rglru: too many chunks");
+    float* carry_a = carry;
+    float* carry_b = carry + size_t(n_seqs) * chunks * width;
+    const dim3 chunk_grid(n_seqs * chunks, scan_grid.y);
+    rglru_chunk_local_kernel<<<chunk_grid, scan_threads, 0, s>>>(a, carry_a, carry_b, chunks);
+    if (dtype == kF32) {
+      rglru_chunk_carry_kernel<float><<<scan_grid, scan_threads, 0, s>>>(a, carry_a, carry_b, chunks);
+      rglru_chunk_apply_kernel<float><<<chunk_grid, scan_threads, 0, s>>>(a, carry_b, chunks);
+    } else {
+      rglru_chunk_carry_kernel<bf16_t><<<scan_grid, scan_threads, 0, s>>>(a, carry_a, carry_b, chunks);
+      rglru_chunk_apply_kernel<bf16_t><<<chunk_grid, scan_threads, 0, s>>>(a, carry_b, chunks);
+    }
+    return check_launch("sp_rglru (scan in chunks)");
+  }
   if (dtype == kF32) rglru_scan_kernel<float><<<scan_grid, scan_threads, 0, s>>>(a);
   else rglru_scan_kernel<bf16_t><<<scan_grid, scan_threads, 0, s>>>(a);
   return check_launch("sp_rglru (scan)");
@@ -285,10 +650,19 @@ extern "C" int sp_retention_takes(int dim, int vdim) {
   return (dim + groups - 1) / groups <= 64;
 }
 
+// float32 numbers of the scratch that a step whose longest portion has max_q_len tokens needs for its walk in chunks
+// (0: every request's tokens are walked one after the other and none is needed).
+extern "C" long long sp_retention_scratch_floats(int heads, int dim, int vdim, int n_seqs, int max_q_len) {
+  if (max_q_len <= kRetentionLongPortion || heads <= 0 || dim <= 0 || vdim <= 0 || vdim > 256) return 0;
+  const int C = retention_chunk_tokens(dim, vdim);
+  if (C == 0) return 0;
+  return (long long)n_seqs * ((max_q_len + C - 1) / C) * heads * dim * vdim;
+}
+
 extern "C" int sp_retention(void* stream, int dtype, const void* proj, long long stride, int q_off, int k_off, int v_off, int g_off,
                             int heads, int dim, int vdim, int rotary_dim, const float* cos_sin, const float* decay, float eps,
                             const int32_t* q_start, const int32_t* q_len, const int32_t* state_slots, float* state, void* out,
-                            int T, int n_seqs) {
+                            int T, int n_seqs, int max_q_len, float* scratch) {
   SP_REQUIRE(heads > 0 && sp_retention_takes(dim, vdim), "sp_retention: no kernel for heads of %d and %d numbers", dim, vdim);
   SP_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= dim && (rotary_dim == 0 || cos_sin),
              "sp_retention: %d numbers cannot turn in a head of %d", rotary_dim, dim);
@@ -302,6 +676,10 @@ extern "C" int sp_retention(void* stream, int dtype, const void* proj, long long
   const int groups = 256 / vdim, rows = (dim + groups - 1) / groups;
   RetentionArgs a = {proj, stride, q_off, k_off, v_off, g_off, heads, dim, vdim, rotary_dim, cos_sin, decay, eps, q_start, q_len,
                      state_slots, state, out, groups};
+  if (scratch && sp_retention_scratch_floats(heads, dim, vdim, n_seqs, max_q_len) > 0) {      // a long portion: its chunks side by side
+    if (dtype == kF32) return launch_retention_chunks<float>((hipStream_t)stream, a, n_seqs, max_q_len, scratch);
+    return launch_retention_chunks<bf16_t>((hipStream_t)stream, a, n_seqs, max_q_len, scratch);
+  }
   const int threads = (groups * vdim + 63) / 64 * 64;
   const size_t lds = size_t(2 * dim + groups * vdim) * sizeof(float);
   if (dtype == kF32) return launch_retention<float>((hipStream_t)stream, a, n_seqs, rows, threads, lds);

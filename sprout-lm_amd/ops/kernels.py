@@ -766,8 +766,10 @@ def rglru_takes(width: int, blocks: int, taps: int) -> bool:
 
 def rglru(proj: torch.Tensor, y_off: int, x_off: int, width: int, blocks: int, taps: int, conv_w, conv_b, wa, ba, wi, bi, lam,
           q_start, q_len, seq_of_token, state_slots, n_seqs: int, state: torch.Tensor, tail, decay: torch.Tensor,
-          drive: torch.Tensor, out: torch.Tensor) -> None:
-    """The gated linear recurrence of sp_rglru (sprout_hip.h) on a step's tokens.  `wa`, `wi`: [blocks, in, out]."""
+          drive: torch.Tensor, out: torch.Tensor, max_q_len: int = 0, workspace=None) -> None:
+    """The gated linear recurrence of sp_rglru (sprout_hip.h) on a step's tokens.  `wa`, `wi`: [blocks, in, out].
+    `max_q_len`: the most tokens one request brings (0: unknown); with `workspace(n)` (a float32 device tensor of at least
+    n elements) long portions are walked in chunks side by side."""
     T, n = out.shape[0], width // max(blocks, 1)
     for t, what in ((proj, "projections"), (out, "recurrence output"), (state, "recurrent state"), (decay, "decay scratch"),
                     (drive, "drive scratch")):
@@ -792,11 +794,17 @@ def rglru(proj: torch.Tensor, y_off: int, x_off: int, width: int, blocks: int, t
     for t in (decay, drive):
         if t.dtype != torch.float32 or t.numel() < T * width:
             raise KernelError("rglru: scratch must hold float32 [T, width]")
+    carry = None
+    need = library().sp_rglru_carry_floats(width, n_seqs, int(max_q_len)) if workspace is not None else 0
+    if need:
+        carry = workspace(need)
+        if carry.dtype != torch.float32 or carry.numel() < need or not carry.is_cuda:
+            raise KernelError("rglru: workspace too small")
     check(library().sp_rglru(_stream(), _code(proj, "projections"), proj.data_ptr(), proj.shape[1], y_off, x_off, width, blocks,
                              taps, conv_w.data_ptr(), conv_b.data_ptr(), wa.data_ptr(), ba.data_ptr(), wi.data_ptr(), bi.data_ptr(),
                              lam.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), seq_of_token.data_ptr(), state_slots.data_ptr(),
                              state.data_ptr(), _ptr(tail) if taps > 1 else None, decay.data_ptr(), drive.data_ptr(),
-                             out.data_ptr(), T, n_seqs))
+                             out.data_ptr(), T, n_seqs, int(max_q_len) if carry is not None else 0, _ptr(carry)))
 
 
 def retention_takes(dim: int, vdim: int) -> bool:
@@ -805,8 +813,9 @@ def retention_takes(dim: int, vdim: int) -> bool:
 
 def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, heads: int, dim: int, vdim: int,
               rotary_dim: int, cos_sin, decay: torch.Tensor, eps: float, q_start, q_len, state_slots, n_seqs: int,
-              state: torch.Tensor, out: torch.Tensor) -> None:
-    """Retention of sp_retention (sprout_hip.h) on a step's tokens; `cos_sin`: rope_table of the step's positions."""
+              state: torch.Tensor, out: torch.Tensor, max_q_len: int = 0, workspace=None) -> None:
+    """Retention of sp_retention (sprout_hip.h) on a step's tokens; `cos_sin`: rope_table of the step's positions.
+    `max_q_len`, `workspace`: as for `rglru`."""
     T = out.shape[0]
     _gpu(proj, "projections"); _gpu(out, "retention output"); _gpu(state, "retention state"); _gpu(decay, "decays")
     if proj.shape[0] < T or out.dtype != proj.dtype or tuple(out.shape) != (T, heads * vdim):
@@ -823,10 +832,16 @@ def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int
             raise KernelError("retention: the rotation table must be float32 [T, rotary_dim / 2, 2]")
     for t, what in ((q_start, "q_start"), (q_len, "q_len"), (state_slots, "state_slots")):
         _ints(t, n_seqs, what)
+    scratch = None
+    need = library().sp_retention_scratch_floats(heads, dim, vdim, n_seqs, int(max_q_len)) if workspace is not None else 0
+    if need:
+        scratch = workspace(need)
+        if scratch.dtype != torch.float32 or scratch.numel() < need or not scratch.is_cuda:
+            raise KernelError("retention: workspace too small")
     check(library().sp_retention(_stream(), _code(proj, "projections"), proj.data_ptr(), proj.shape[1], q_off, k_off, v_off, g_off,
                                  heads, dim, vdim, rotary_dim, _ptr(cos_sin) if rotary_dim else None, decay.data_ptr(), float(eps),
                                  q_start.data_ptr(), q_len.data_ptr(), state_slots.data_ptr(), state.data_ptr(), out.data_ptr(),
-                                 T, n_seqs))
+                                 T, n_seqs, int(max_q_len) if scratch is not None else 0, _ptr(scratch)))
 
 
 def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm_weight=None, eps: float = 0.0,

@@ -43,10 +43,10 @@ def _declare(lib):
         "sp_scaled_add": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_float, c_int, c_int],
         "sp_head_gate": [c_void, c_int, c_void, c_void, c_i64, c_int, c_int, c_int],
         "sp_rglru_takes": [c_int] * 3,
-        "sp_rglru": [c_void, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_int] + [c_void] * 16 + [c_int, c_int],
+        "sp_rglru": [c_void, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_int] + [c_void] * 16 + [c_int, c_int, c_int, c_void],
         "sp_retention_takes": [c_int] * 2,
         "sp_retention": [c_void, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_void,
-                         c_float, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
+                         c_float, c_void, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "sp_gate_up_silu": [c_void, c_void, c_void, c_int, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int, c_float, c_void, c_i64],
         "sp_gate_up_silu_f32_takes": [c_int, c_int, c_int],
         "sp_gate_up_silu_f32": [c_void, c_void, c_void, c_float, c_void, c_void, c_int, c_int, c_int, c_int, c_float, c_void, c_i64],
@@ -85,6 +85,10 @@ def _declare(lib):
     }
     lib.sp_attention_workspace_floats.argtypes = [c_int] * 10
     lib.sp_attention_workspace_floats.restype = c_i64
+    lib.sp_rglru_carry_floats.argtypes = [c_int] * 3
+    lib.sp_rglru_carry_floats.restype = c_i64
+    lib.sp_retention_scratch_floats.argtypes = [c_int] * 5
+    lib.sp_retention_scratch_floats.restype = c_i64
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
         fn.argtypes = argtypes

@@ -82,5 +82,6 @@ class GatedLinearRecurrence(Mixer):
         out = ctx.buffer("recurrence_out", (T, W), ctx.act_dtype)
         ops.rglru(proj, 0, W, W, self.blocks, self.taps, self.conv_w, self.conv_b, self.w_a, self.b_a, self.w_i, self.b_i,
                   self.lam, ctx.q_start, ctx.q_len, ctx.seq_of_token, ctx.state_slots, ctx.n_seqs, cache["state"].state,
-                  cache["inputs"].state if self.taps > 1 else None, scratch[0], scratch[1], out)
+                  cache["inputs"].state if self.taps > 1 else None, scratch[0], scratch[1], out, max_q_len=ctx.max_q_len,
+                  workspace=lambda n: ctx.buffer("recurrence_carry", (n,), torch.float32))
         ops.gemm(out, self.w_o, residual, accumulate=True)

@@ -81,5 +81,6 @@ class Retention(Mixer):
         table = self.position.table(ctx) if rotary else None
         out = ctx.buffer("retention_out", (T, H * V), ctx.act_dtype)
         ops.retention(proj, 0, H * D, 2 * H * D, 2 * H * D + H * V, H, D, V, rotary, table, self.decays, self.eps,
-                      ctx.q_start, ctx.q_len, ctx.state_slots, ctx.n_seqs, cache.state, out)
+                      ctx.q_start, ctx.q_len, ctx.state_slots, ctx.n_seqs, cache.state, out, max_q_len=ctx.max_q_len,
+                      workspace=lambda n: ctx.buffer("retention_chunks", (n,), torch.float32))
         ops.gemm(out, self.w_o, residual, accumulate=True)
