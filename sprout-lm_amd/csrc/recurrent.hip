@@ -40,12 +40,15 @@ struct LruArgs {
   int T;
 };
 
-// A block takes TT tokens of one diagonal block of channels: their convolution outputs wait in LDS, then every thread
-// owns output channels of both gates and walks the block's inputs once for all TT tokens.
+// A block takes TT tokens of one diagonal block of channels: their convolution outputs wait in LDS; then a thread owns
+// an output channel of both gates and one of `slices` equal shares of the block's inputs (256 threads = lanes x slices),
+// walks its share once for all TT tokens, and the slices' sums meet in LDS.
 template <typename T, int TT>
-__global__ __launch_bounds__(256) void rglru_gates_kernel(LruArgs a) {
-  extern __shared__ float u_s[];      // [TT][n]
+__global__ __launch_bounds__(256) void rglru_gates_kernel(LruArgs a, int lanes) {
+  extern __shared__ float u_s[];      // [TT][n], then the slices' sums [slices - 1][TT][2][lanes]
   const int n = a.width / a.blocks, b = blockIdx.y, t0 = blockIdx.x * TT, c0 = b * n;
+  const int slices = blockDim.x / lanes, lane = threadIdx.x % lanes, slice = threadIdx.x / lanes;
+  float* sums = u_s + TT * n;
   const T* proj = (const T*)a.proj;
   const int keep = a.taps - 1;
   for (int e = threadIdx.x; e < TT * n; e += blockDim.x) {
@@ -66,30 +69,57 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(LruArgs a) {
     u_s[e] = u;
   }
   __syncthreads();
-  for (int o = threadIdx.x; o < n; o += blockDim.x) {
+  const int share = (n + slices - 1) / slices, k_first = slice * share, k_end = min(n, k_first + share);
+  for (int o0 = 0; o0 < n; o0 += lanes) {
+    const int o = o0 + lane;
+    const bool live = o < n;
     float ra[TT], ri[TT];
-    const float bias_a = to_float(((const T*)a.ba)[c0 + o]), bias_i = to_float(((const T*)a.bi)[c0 + o]);
 #pragma unroll
-    for (int tt = 0; tt < TT; ++tt) { ra[tt] = bias_a; ri[tt] = bias_i; }
-    const T* wa = (const T*)a.wa + size_t(b) * n * n + o;
-    const T* wi = (const T*)a.wi + size_t(b) * n * n + o;
-    for (int k = 0; k < n; ++k) {
-      const float va = to_float(wa[size_t(k) * n]), vi = to_float(wi[size_t(k) * n]);
+    for (int tt = 0; tt < TT; ++tt) ra[tt] = ri[tt] = 0.f;
+    if (live) {
+      const T* wa = (const T*)a.wa + size_t(b) * n * n + o;
+      const T* wi = (const T*)a.wi + size_t(b) * n * n + o;
+#pragma unroll 8
+      for (int k = k_first; k < k_end; ++k) {
+        const float va = to_float(wa[size_t(k) * n]), vi = to_float(wi[size_t(k) * n]);
 #pragma unroll
-      for (int tt = 0; tt < TT; ++tt) {
-        const float u = u_s[tt * n + k];
-        ra[tt] = fmaf(va, u, ra[tt]);
-        ri[tt] = fmaf(vi, u, ri[tt]);
+        for (int tt = 0; tt < TT; ++tt) {
+          const float u = u_s[tt * n + k];
+          ra[tt] = fmaf(va, u, ra[tt]);
+          ri[tt] = fmaf(vi, u, ri[tt]);
+        }
       }
     }
+    if (slices > 1) {
+      if (o0) __syncthreads();      // the sums of the channels before have been read
+      if (slice) {
+        float* mine = sums + size_t(slice - 1) * TT * 2 * lanes + lane;
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+          mine[(2 * tt) * lanes] = ra[tt];
+          mine[(2 * tt + 1) * lanes] = ri[tt];
+        }
+      }
+      __syncthreads();
+    }
+    if (slice || !live) continue;
+    for (int other = 1; other < slices; ++other) {
+      const float* theirs = sums + size_t(other - 1) * TT * 2 * lanes + lane;
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) {
+        ra[tt] += theirs[(2 * tt) * lanes];
+        ri[tt] += theirs[(2 * tt + 1) * lanes];
+      }
+    }
+    const float bias_a = to_float(((const T*)a.ba)[c0 + o]), bias_i = to_float(((const T*)a.bi)[c0 + o]);
     const float rate = 8.0f * softplus(to_float(((const T*)a.lam)[c0 + o]));
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) {
       const int t = t0 + tt;
       if (t >= a.T) break;
-      const float log_a = -rate * sigmoid(ra[tt]);
+      const float log_a = -rate * sigmoid(ra[tt] + bias_a);
       a.decay[size_t(t) * a.width + c0 + o] = expf(log_a);
-      a.drive[size_t(t) * a.width + c0 + o] = sqrtf(-expm1f(2.0f * log_a)) * sigmoid(ri[tt]) * u_s[tt * n + o];
+      a.drive[size_t(t) * a.width + c0 + o] = sqrtf(-expm1f(2.0f * log_a)) * sigmoid(ri[tt] + bias_i) * u_s[tt * n + o];
     }
   }
 }
@@ -398,10 +428,23 @@ __global__ __launch_bounds__(256) void retention_chunk_carry_kernel(RetentionArg
   const float gamma = a.decay[h];
   float* kept = a.state + (size_t(slot) * a.heads + h) * DV + e;
   float S = *kept;
-  for (int ci = 0; ci < used; ++ci) {
-    float* at = scratch + ((size_t(s) * chunks + ci) * a.heads + h) * DV + e;
+  const size_t step = size_t(a.heads) * DV;
+  float* at = scratch + (size_t(s) * chunks * a.heads + h) * DV + e;
+  const float whole = powf(gamma, float(C));
+  int ci = 0;
+  for (; ci + 8 <= used && (ci + 8) * C <= n; ci += 8, at += 8 * step) {      // eight whole chunks: their sums are asked for together
+    float U[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) U[j] = at[j * step];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      at[j * step] = S;          // what the chunk starts from
+      S = fmaf(whole, S, U[j]);
+    }
+  }
+  for (; ci < used; ++ci, at += step) {
     const float U = *at;
-    *at = S;          // what the chunk starts from
+    *at = S;
     S = fmaf(powf(gamma, float(min(C, n - ci * C))), S, U);
   }
   *kept = S;
@@ -607,15 +650,16 @@ extern "C" int sp_rglru(void* stream, int dtype, const void* proj, long long str
                state_slots, state, tail, decay, drive, out, T};
   hipStream_t s = (hipStream_t)stream;
   const int n = width / blocks;
-  const int tt = T <= 1 ? 1 : (T <= 8 || n > 512) ? 4 : 16;      // a tile's convolution outputs stay within 32 KB of LDS
-  const int threads = n >= 256 ? 256 : (n + 63) / 64 * 64;
+  // few tokens: a block each, so that the chip has blocks enough; a tile's convolution outputs and sums stay within 40 KB of LDS
+  const int tt = T <= 16 ? 1 : (T <= 64 || n > 512) ? 4 : 16;
+  const int lanes = n >= 256 ? 256 : n > 64 ? 128 : 64, slices = 256 / lanes;
   const dim3 grid((T + tt - 1) / tt, blocks);
-  const size_t lds = size_t(tt) * n * sizeof(float);
+  const size_t lds = (size_t(tt) * n + size_t(slices - 1) * tt * 2 * lanes) * sizeof(float);
 #define SP_GATES(TYPE)                                                                        \
   do {                                                                                        \
-    if (tt == 1) rglru_gates_kernel<TYPE, 1><<<grid, threads, lds, s>>>(a);                   \
-    else if (tt == 4) rglru_gates_kernel<TYPE, 4><<<grid, threads, lds, s>>>(a);              \
-    else rglru_gates_kernel<TYPE, 16><<<grid, threads, lds, s>>>(a);                          \
+    if (tt == 1) rglru_gates_kernel<TYPE, 1><<<grid, 256, lds, s>>>(a, lanes);                \
+    else if (tt == 4) rglru_gates_kernel<TYPE, 4><<<grid, 256, lds, s>>>(a, lanes);           \
+    else rglru_gates_kernel<TYPE, 16><<<grid, 256, lds, s>>>(a, lanes);                       \
   } while (0)
   if (dtype == kF32) SP_GATES(float);
   else SP_GATES(bf16_t);
