@@ -58,7 +58,7 @@ GENERAL = model(128, 300, [
     layer(rglru(192, 2, 3), 96),
     layer(retention(2, 32, 64, (0.9, 0.995), rot(32, 1000.0)), 64),
     layer(attention(16, 1, 64, 32, 0.1, rot(32, 250.0, (8.0, 64, 16.0, 1.0))), 96),
-    layer(retention(4, 64, 16, (0.96875, 0.99, 0.999, 0.9999), rot(16, 1e6))),
+    layer(retention(4, 64, 16, (0.95, 0.99, 0.999, 0.9999), rot(16, 1e6))),
     layer(rglru(128, 8, 2), 32),
 ], mult=0.6, logit_scale=0.5)
 # no attention at all: a model whose requests hold no pages, only state slots
