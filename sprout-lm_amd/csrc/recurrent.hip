@@ -363,6 +363,54 @@ __device__ __forceinline__ float turned(const T* src, const float* cos_sin, size
   return to_float(src[d]);
 }
 
+// Heads too large for the registers of one block: the state stays in memory.  A thread owns columns v, v + 256, ... of the
+// head's state, walks their rows for every token (S <- decay S + k v^T and the column's sum S^T q in one pass), and the
+// head's unit norm needs the columns' sums only.  Any dim and vdim; slow, for sizes the other kernel does not take.
+template <typename T>
+__global__ __launch_bounds__(256) void retention_general_kernel(RetentionArgs a) {
+  extern __shared__ float lds[];      // q [dim], k [dim], the columns' sums [vdim]
+  __shared__ float scratch[16];
+  const int s = blockIdx.x, h = blockIdx.y, D = a.dim, V = a.vdim, half = a.rotary_dim / 2;
+  float* qs = lds;
+  float* ks = lds + D;
+  float* o_row = lds + 2 * D;
+  const int start = a.q_start[s], n = a.q_len[s], slot = a.state_slots[s];
+  float* kept = a.state + (size_t(slot) * a.heads + h) * D * V;
+  const float gamma = a.decay[h], k_scale = 1.0f / sqrtf(float(D));
+  const T* proj = (const T*)a.proj;
+  T* out = (T*)a.out;
+  for (int t = start; t < start + n; ++t) {
+    const T* row = proj + size_t(t) * a.stride;
+    for (int i = threadIdx.x; i < 2 * D; i += blockDim.x) {
+      const bool is_k = i >= D;
+      const int d = is_k ? i - D : i;
+      const float value = turned(row + (is_k ? a.k_off : a.q_off) + h * D, a.cos_sin, size_t(t), d, half);
+      if (is_k) ks[d] = value * k_scale;
+      else qs[d] = value;
+    }
+    __syncthreads();
+    float squares = 0.f;
+    for (int v = threadIdx.x; v < V; v += blockDim.x) {
+      const float value = to_float(row[a.v_off + h * V + v]);
+      float o = 0.f;
+      for (int d = 0; d < D; ++d) {
+        const float S = fmaf(gamma, kept[size_t(d) * V + v], ks[d] * value);
+        kept[size_t(d) * V + v] = S;
+        o = fmaf(S, qs[d], o);
+      }
+      o_row[v] = o;
+      squares = fmaf(o, o, squares);
+    }
+    squares = block_sum(squares, scratch);
+    const float unit = 1.0f / sqrtf(squares / float(V) + a.eps);
+    for (int v = threadIdx.x; v < V; v += blockDim.x) {      // a thread reads back what it wrote itself
+      const float g = to_float(row[a.g_off + h * V + v]);
+      out[(size_t(t) * a.heads + h) * V + v] = from_float<T>((o_row[v] * unit) * (g * sigmoid(g)));
+    }
+    __syncthreads();
+  }
+}
+
 template <typename T, int CV>
 __global__ __launch_bounds__(256) void retention_chunk_local_kernel(RetentionArgs a, float* __restrict__ scratch, int chunks, int C) {
   extern __shared__ float lds[];      // k [C][D + 1] (times its power of the decay), v [C][V]
@@ -688,10 +736,15 @@ extern "C" int sp_rglru(void* stream, int dtype, const void* proj, long long str
   return check_launch("sp_rglru (scan)");
 }
 
-extern "C" int sp_retention_takes(int dim, int vdim) {
-  if (dim <= 0 || vdim <= 0 || vdim > 256) return 0;
+// Whether a head's state fits the registers of one block (a thread: one column, at most 64 rows).
+static bool retention_in_registers(int dim, int vdim) {
+  if (vdim > 256) return false;
   const int groups = 256 / vdim;
   return (dim + groups - 1) / groups <= 64;
+}
+
+extern "C" int sp_retention_takes(int dim, int vdim) {
+  return dim > 0 && vdim > 0 && (retention_in_registers(dim, vdim) || size_t(2 * dim + vdim) * sizeof(float) <= 64 * 1024);
 }
 
 // float32 numbers of the scratch that a step whose longest portion has max_q_len tokens needs for its walk in chunks
@@ -717,12 +770,19 @@ extern "C" int sp_retention(void* stream, int dtype, const void* proj, long long
   SP_REQUIRE(proj && decay && q_start && q_len && state_slots && state && out, "sp_retention: null operand");
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_retention: unsupported dtype %d", dtype);
   if (T == 0 || n_seqs == 0) return 0;
-  const int groups = 256 / vdim, rows = (dim + groups - 1) / groups;
+  const int groups = vdim <= 256 ? 256 / vdim : 1, rows = (dim + groups - 1) / groups;
   RetentionArgs a = {proj, stride, q_off, k_off, v_off, g_off, heads, dim, vdim, rotary_dim, cos_sin, decay, eps, q_start, q_len,
                      state_slots, state, out, groups};
   if (scratch && sp_retention_scratch_floats(heads, dim, vdim, n_seqs, max_q_len) > 0) {      // a long portion: its chunks side by side
     if (dtype == kF32) return launch_retention_chunks<float>((hipStream_t)stream, a, n_seqs, max_q_len, scratch);
     return launch_retention_chunks<bf16_t>((hipStream_t)stream, a, n_seqs, max_q_len, scratch);
+  }
+  if (!retention_in_registers(dim, vdim)) {
+    const size_t general_lds = size_t(2 * dim + vdim) * sizeof(float);
+    const dim3 grid(n_seqs, heads);
+    if (dtype == kF32) retention_general_kernel<float><<<grid, 256, general_lds, (hipStream_t)stream>>>(a);
+    else retention_general_kernel<bf16_t><<<grid, 256, general_lds, (hipStream_t)stream>>>(a);
+    return check_launch("sp_retention (state in memory)");
   }
   const int threads = (groups * vdim + 63) / 64 * 64;
   const size_t lds = size_t(2 * dim + groups * vdim) * sizeof(float);

@@ -215,7 +215,7 @@ def test_recurrence_keeps_a_far_token():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,dim,vdim,dims", [(3, 20, 6, 8), (2, 32, 64, 32), (4, 64, 16, 16), (2, 10, 30, 0), (1, 128, 128, 64),
-                                                  (2, 256, 64, 32), (2, 48, 200, 48)])
+                                                  (2, 256, 64, 32), (2, 48, 200, 48), (1, 130, 256, 64), (2, 24, 300, 0)])
 def test_retention_alone_in_portions(dtype, heads, dim, vdim, dims):
     from sprout_lm_amd.models.plan import PartPlan
     rng = np.random.default_rng(dim + vdim)
