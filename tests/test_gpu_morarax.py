@@ -431,6 +431,22 @@ def test_replay_with_other_page_sizes(folders, name, page, dtype):
     check(folders[name], dtype, requests, trace, results)
 
 
+@pytest.mark.parametrize("name,dtype", [("general", "float32"), ("states", "float32"), ("odd", "bfloat16")])
+def test_long_prompts_in_long_portions(folders, name, dtype):
+    """Prompts of many chunks of the recurrent mixers' long-portion kernels: whole, in long uneven portions (chunk edges
+    fall anywhere), and two requests' long portions beside each other and beside single tokens."""
+    requests = requests_for(name, [700, 333], seed=500)
+    cut = traces.portions(requests, sizes=(200, 129, 65, 2, 64, 190, 1, 70))
+    both = traces.Trace()
+    a, b = requests["r0"], requests["r1"]
+    both.add([("r0", 0, a[:400], range(390, 400)), ("r1", 0, b[:150], [149])])
+    both.add([("r0", 400, a[400:401], [0]), ("r1", 150, b[150:], range(0, 183, 7))], end=["r1"])
+    both.add([("r0", 401, a[401:], range(0, 299, 5))], end=["r0"])
+    for trace in (traces.whole(requests), cut, both):
+        results = replay(folders[name], name, dtype, trace, 1280)
+        check(folders[name], dtype, requests, trace, results)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_cuts_agree_with_each_other(folders, dtype):
     """Whole, token-by-token and portioned replays give the same logits beyond rounding."""
