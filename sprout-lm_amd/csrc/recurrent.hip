@@ -40,24 +40,33 @@ struct LruArgs {
   int T;
 };
 
-// A block takes TT tokens of one diagonal block of channels: their convolution outputs wait in LDS; then a thread owns
-// an output channel of both gates and one of `slices` equal shares of the block's inputs (256 threads = lanes x slices),
-// walks its share once for all TT tokens, and the slices' sums meet in LDS.
+// The convolution outputs of TT tokens from t0 on, channels c0 .. c0 + n - 1, into u_s [TT][n].  Where a token lies in its
+// request's share of the step and which state row is its request's is looked up once per token, not once per channel, so
+// that the channels' loads do not each wait behind that chain.
 template <typename T, int TT>
-__global__ __launch_bounds__(256) void rglru_gates_kernel(LruArgs a, int lanes) {
-  extern __shared__ float u_s[];      // [TT][n], then the slices' sums [slices - 1][TT][2][lanes]
-  const int n = a.width / a.blocks, b = blockIdx.y, t0 = blockIdx.x * TT, c0 = b * n;
-  const int slices = blockDim.x / lanes, lane = threadIdx.x % lanes, slice = threadIdx.x / lanes;
-  float* sums = u_s + TT * n;
+__device__ __forceinline__ void conv_outputs(const LruArgs& a, float* u_s, int t0, int c0, int n) {
+  __shared__ int place[TT], row[TT];
+  if (threadIdx.x < TT) {
+    const int t = t0 + threadIdx.x;
+    int j = 0, slot = 0;
+    if (t < a.T) {
+      const int s = a.seq_of_token[t];
+      j = t - a.q_start[s];
+      slot = a.state_slots[s];
+    }
+    place[threadIdx.x] = j;
+    row[threadIdx.x] = slot;
+  }
+  __syncthreads();
   const T* proj = (const T*)a.proj;
   const int keep = a.taps - 1;
+#pragma unroll 4
   for (int e = threadIdx.x; e < TT * n; e += blockDim.x) {
     const int tt = e / n, c = c0 + e % n, t = t0 + tt;
     float u = 0.f;
     if (t < a.T) {
-      const int s = a.seq_of_token[t];
-      const int j = t - a.q_start[s];      // the token's place in its request's share of the step
-      const float* tail = a.tail + size_t(a.state_slots[s]) * keep * a.width;
+      const int j = place[tt];
+      const float* tail = a.tail + size_t(row[tt]) * keep * a.width;
       u = to_float(((const T*)a.conv_b)[c]);
       for (int tap = 0; tap < a.taps; ++tap) {
         const int back = keep - tap;
@@ -69,6 +78,18 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(LruArgs a, int lanes) 
     u_s[e] = u;
   }
   __syncthreads();
+}
+
+// A block takes TT tokens of one diagonal block of channels: their convolution outputs wait in LDS; then a thread owns
+// an output channel of both gates and one of `slices` equal shares of the block's inputs (256 threads = lanes x slices),
+// walks its share once for all TT tokens, and the slices' sums meet in LDS.
+template <typename T, int TT>
+__global__ __launch_bounds__(256) void rglru_gates_kernel(LruArgs a, int lanes) {
+  extern __shared__ float u_s[];      // [TT][n], then the slices' sums [slices - 1][TT][2][lanes]
+  const int n = a.width / a.blocks, b = blockIdx.y, t0 = blockIdx.x * TT, c0 = b * n;
+  const int slices = blockDim.x / lanes, lane = threadIdx.x % lanes, slice = threadIdx.x / lanes;
+  float* sums = u_s + TT * n;
+  conv_outputs<T, TT>(a, u_s, t0, c0, n);
   const int share = (n + slices - 1) / slices, k_first = slice * share, k_end = min(n, k_first + share);
   for (int o0 = 0; o0 < n; o0 += lanes) {
     const int o = o0 + lane;
@@ -79,8 +100,25 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(LruArgs a, int lanes) 
     if (live) {
       const T* wa = (const T*)a.wa + size_t(b) * n * n + o;
       const T* wi = (const T*)a.wi + size_t(b) * n * n + o;
-#pragma unroll 8
-      for (int k = k_first; k < k_end; ++k) {
+      int k = k_first;
+      if ((n & 3) == 0 && (k_first & 3) == 0) {      // four inputs at a time: a token's four convolution outputs in one LDS read
+#pragma unroll 2
+        for (; k + 4 <= k_end; k += 4) {
+          float va[4], vi[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            va[j] = to_float(wa[size_t(k + j) * n]);
+            vi[j] = to_float(wi[size_t(k + j) * n]);
+          }
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) {
+            const float4 u = *reinterpret_cast<const float4*>(u_s + tt * n + k);
+            ra[tt] = fmaf(va[3], u.w, fmaf(va[2], u.z, fmaf(va[1], u.y, fmaf(va[0], u.x, ra[tt]))));
+            ri[tt] = fmaf(vi[3], u.w, fmaf(vi[2], u.z, fmaf(vi[1], u.y, fmaf(vi[0], u.x, ri[tt]))));
+          }
+        }
+      }
+      for (; k < k_end; ++k) {
         const float va = to_float(wa[size_t(k) * n]), vi = to_float(wi[size_t(k) * n]);
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
@@ -121,6 +159,92 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(LruArgs a, int lanes) 
       a.decay[size_t(t) * a.width + c0 + o] = expf(log_a);
       a.drive[size_t(t) * a.width + c0 + o] = sqrtf(-expm1f(2.0f * log_a)) * sigmoid(ri[tt] + bias_i) * u_s[tt * n + o];
     }
+  }
+}
+
+// The gates of a few tokens (a decode step) in bfloat16 storage: what counts is how soon the block's two matrices have
+// come from memory.  A thread asks for eight neighbouring outputs of an input at a time (16 bytes), n / 8 threads cover an
+// input's row, the block's threads beyond that share the inputs in slices; a thread's loads do not wait for each other.
+template <int TT>
+__global__ __launch_bounds__(256) void rglru_gates_few_kernel(LruArgs a, int slices) {
+  extern __shared__ float u_s[];      // [TT][n], then the slices' sums [slices][TT][2][n]
+  using T = bf16_t;
+  constexpr int KB = 8;               // inputs whose rows a thread asks for at once
+  const int n = a.width / a.blocks, b = blockIdx.y, t0 = blockIdx.x * TT, c0 = b * n, cols = n / 8;
+  float* sums = u_s + TT * n;
+  const int col = threadIdx.x % cols, slice = threadIdx.x / cols;
+  const int share = (n + slices - 1) / slices, k_first = slice * share, k_end = slice < slices ? min(n, k_first + share) : 0;
+  const T* wa = (const T*)a.wa + size_t(b) * n * n + col * 8;
+  const T* wi = (const T*)a.wi + size_t(b) * n * n + col * 8;
+  uint4 pa[KB], pi[KB];
+#pragma unroll
+  for (int j = 0; j < KB; ++j) {      // the first rows are on their way while the convolution is taken
+    const bool in = k_first + j < k_end;
+    pa[j] = in ? *reinterpret_cast<const uint4*>(wa + size_t(k_first + j) * n) : uint4{0, 0, 0, 0};
+    pi[j] = in ? *reinterpret_cast<const uint4*>(wi + size_t(k_first + j) * n) : uint4{0, 0, 0, 0};
+  }
+  // what the first output of this thread in the last stage needs, likewise
+  const int o_first = threadIdx.x % n;
+  const bool ends = threadIdx.x < TT * n;
+  const float bias_a0 = ends ? to_float(((const T*)a.ba)[c0 + o_first]) : 0.f;
+  const float bias_i0 = ends ? to_float(((const T*)a.bi)[c0 + o_first]) : 0.f;
+  const float lam0 = ends ? to_float(((const T*)a.lam)[c0 + o_first]) : 0.f;
+  conv_outputs<T, TT>(a, u_s, t0, c0, n);
+  if (slice < slices) {
+    float ra[TT][8], ri[TT][8];
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ra[tt][j] = ri[tt][j] = 0.f;
+    for (int kb = k_first; kb < k_end; kb += KB) {
+      if (kb != k_first) {
+#pragma unroll
+        for (int j = 0; j < KB; ++j) {
+          const bool in = kb + j < k_end;
+          pa[j] = in ? *reinterpret_cast<const uint4*>(wa + size_t(kb + j) * n) : uint4{0, 0, 0, 0};
+          pi[j] = in ? *reinterpret_cast<const uint4*>(wi + size_t(kb + j) * n) : uint4{0, 0, 0, 0};
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < KB; ++j) {
+        const int k = min(kb + j, n - 1);      // rows past the share hold zeros
+        const uint32_t wa2[4] = {pa[j].x, pa[j].y, pa[j].z, pa[j].w}, wi2[4] = {pi[j].x, pi[j].y, pi[j].z, pi[j].w};
+#pragma unroll
+        for (int tt = 0; tt < TT; ++tt) {
+          const float u = u_s[tt * n + k];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            ra[tt][2 * q] = fmaf(__uint_as_float(wa2[q] << 16), u, ra[tt][2 * q]);
+            ra[tt][2 * q + 1] = fmaf(__uint_as_float(wa2[q] & 0xffff0000u), u, ra[tt][2 * q + 1]);
+            ri[tt][2 * q] = fmaf(__uint_as_float(wi2[q] << 16), u, ri[tt][2 * q]);
+            ri[tt][2 * q + 1] = fmaf(__uint_as_float(wi2[q] & 0xffff0000u), u, ri[tt][2 * q + 1]);
+          }
+        }
+      }
+    }
+    float* mine = sums + size_t(slice) * TT * 2 * n + col * 8;
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        mine[(2 * tt) * n + j] = ra[tt][j];
+        mine[(2 * tt + 1) * n + j] = ri[tt][j];
+      }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < TT * n; e += blockDim.x) {
+    const int tt = e / n, o = e % n, t = t0 + tt;
+    if (t >= a.T) continue;
+    const bool first = e == threadIdx.x;
+    float ra = first ? bias_a0 : to_float(((const T*)a.ba)[c0 + o]), ri = first ? bias_i0 : to_float(((const T*)a.bi)[c0 + o]);
+    for (int other = 0; other < slices; ++other) {
+      ra += sums[(size_t(other) * TT * 2 + 2 * tt) * n + o];
+      ri += sums[(size_t(other) * TT * 2 + 2 * tt + 1) * n + o];
+    }
+    const float rate = 8.0f * softplus(first ? lam0 : to_float(((const T*)a.lam)[c0 + o]));
+    const float log_a = -rate * sigmoid(ra);
+    a.decay[size_t(t) * a.width + c0 + o] = expf(log_a);
+    a.drive[size_t(t) * a.width + c0 + o] = sqrtf(-expm1f(2.0f * log_a)) * sigmoid(ri) * u_s[tt * n + o];
   }
 }
 
@@ -295,6 +419,9 @@ __global__ __launch_bounds__(256) void retention_kernel(RetentionArgs a) {
   T* out = (T*)a.out;
   for (int t = start; t < start + n; ++t) {
     const T* row = proj + size_t(t) * a.stride;
+    // the value and the gate are asked for here, before the waits on the block: their way from memory is not waited for twice
+    const float value_v = active ? to_float(row[a.v_off + h * V + v]) : 0.f;
+    const float g = threadIdx.x < V ? to_float(row[a.g_off + h * V + threadIdx.x]) : 0.f;
     for (int i = threadIdx.x; i < 2 * D; i += blockDim.x) {
       const bool is_k = i >= D;
       const int d = is_k ? i - D : i;
@@ -314,12 +441,11 @@ __global__ __launch_bounds__(256) void retention_kernel(RetentionArgs a) {
     __syncthreads();
     float partial = 0.f;
     if (active) {
-      const float value = to_float(row[a.v_off + h * V + v]);
 #pragma unroll
       for (int r = 0; r < ROWS; ++r) {
         const int d = dr + r * R;
         if (d < D) {
-          S[r] = fmaf(gamma, S[r], ks[d] * value);
+          S[r] = fmaf(gamma, S[r], ks[d] * value_v);
           partial = fmaf(S[r], qs[d], partial);
         }
       }
@@ -331,7 +457,6 @@ __global__ __launch_bounds__(256) void retention_kernel(RetentionArgs a) {
       for (int j = 0; j < R; ++j) o += part[j * V + threadIdx.x];
     const float squares = block_sum(o * o, scratch);
     if (threadIdx.x < V) {
-      const float g = to_float(row[a.g_off + h * V + threadIdx.x]);
       const float unit = 1.0f / sqrtf(squares / float(V) + a.eps);
       out[(size_t(t) * a.heads + h) * V + threadIdx.x] = from_float<T>((o * unit) * (g * sigmoid(g)));
     }
@@ -700,18 +825,33 @@ extern "C" int sp_rglru(void* stream, int dtype, const void* proj, long long str
   const int n = width / blocks;
   // few tokens: a block each, so that the chip has blocks enough; a tile's convolution outputs and sums stay within 40 KB of LDS
   const int tt = T <= 16 ? 1 : (T <= 64 || n > 512) ? 4 : 16;
-  const int lanes = n >= 256 ? 256 : n > 64 ? 128 : 64, slices = 256 / lanes;
+  bool wide = false;
+  if (dtype == kBF16 && tt <= 4 && n % 8 == 0 && n / 8 <= 256) {      // few tokens: the matrices sixteen bytes at a time
+    const int cols = n / 8, few_slices = min(256 / cols, tt == 1 ? 16 : 8);
+    const size_t few_lds = (size_t(tt) * n + size_t(few_slices) * tt * 2 * n) * sizeof(float);
+    if (few_lds <= 48 * 1024) {
+      const dim3 few_grid((T + tt - 1) / tt, blocks);
+      if (tt == 1) rglru_gates_few_kernel<1><<<few_grid, 256, few_lds, s>>>(a, few_slices);
+      else rglru_gates_few_kernel<4><<<few_grid, 256, few_lds, s>>>(a, few_slices);
+      wide = true;
+    }
+  }
+  if (!wide) {
+  // many tokens: a thread an output, all of the block's inputs; fewer: the inputs in slices over 256 threads
+  const int lanes = n >= 256 ? 256 : tt == 16 ? (n + 63) / 64 * 64 : n > 64 ? 128 : 64, slices = tt == 16 ? 1 : 256 / lanes;
+  const int threads = lanes * slices;
   const dim3 grid((T + tt - 1) / tt, blocks);
   const size_t lds = (size_t(tt) * n + size_t(slices - 1) * tt * 2 * lanes) * sizeof(float);
 #define SP_GATES(TYPE)                                                                        \
   do {                                                                                        \
-    if (tt == 1) rglru_gates_kernel<TYPE, 1><<<grid, 256, lds, s>>>(a, lanes);                \
-    else if (tt == 4) rglru_gates_kernel<TYPE, 4><<<grid, 256, lds, s>>>(a, lanes);           \
-    else rglru_gates_kernel<TYPE, 16><<<grid, 256, lds, s>>>(a, lanes);                       \
+    if (tt == 1) rglru_gates_kernel<TYPE, 1><<<grid, threads, lds, s>>>(a, lanes);              \
+    else if (tt == 4) rglru_gates_kernel<TYPE, 4><<<grid, threads, lds, s>>>(a, lanes);          \
+    else rglru_gates_kernel<TYPE, 16><<<grid, threads, lds, s>>>(a, lanes);                      \
   } while (0)
   if (dtype == kF32) SP_GATES(float);
   else SP_GATES(bf16_t);
 #undef SP_GATES
+  }
   if (check_launch("sp_rglru (gates)")) return 1;
   const int scan_threads = width >= 256 ? 256 : (width + 63) / 64 * 64;
   const dim3 scan_grid(n_seqs, (width + scan_threads - 1) / scan_threads);
