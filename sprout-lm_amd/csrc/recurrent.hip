@@ -289,7 +289,8 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(LruArgs a) {
 // The same walk for long portions, in three passes over chunks of kScanChunk tokens so that a request's tokens are shared
 // out over the chip: every chunk's own product of decays and its sum from zero; per channel the few chunks one after the
 // other, which leaves every chunk the state it starts from (and the request its new state and convolution inputs); then
-// every chunk again from that state, writing the output.  carry_a, carry_b: float32 [requests * chunks, width].
+// every chunk again from that state, writing the output.  carry_a, carry_b: float32 [T / kScanChunk + requests, width]; chunk ci
+// of request s has row q_start[s] / kScanChunk + s + ci, which keeps unequal requests' rows apart without gaps to speak of.
 constexpr int kScanChunk = 64;
 
 __global__ __launch_bounds__(256) void rglru_chunk_local_kernel(LruArgs a, float* __restrict__ carry_a,
@@ -318,8 +319,9 @@ __global__ __launch_bounds__(256) void rglru_chunk_local_kernel(LruArgs a, float
     B = fmaf(d, B, a.drive[size_t(t) * a.width + c]);
     A *= d;
   }
-  carry_a[size_t(blockIdx.x) * a.width + c] = A;
-  carry_b[size_t(blockIdx.x) * a.width + c] = B;
+  const size_t at = size_t(a.q_start[s] / kScanChunk + s + ci) * a.width + c;
+  carry_a[at] = A;
+  carry_b[at] = B;
 }
 
 template <typename T>
@@ -331,7 +333,7 @@ __global__ __launch_bounds__(256) void rglru_chunk_carry_kernel(LruArgs a, const
   const int used = (n + kScanChunk - 1) / kScanChunk;
   float S = a.state[size_t(slot) * a.width + c];
   for (int ci = 0; ci < used; ++ci) {
-    const size_t at = (size_t(s) * chunks + ci) * a.width + c;
+    const size_t at = (size_t(start / kScanChunk + s) + ci) * a.width + c;
     const float A = carry_a[at], B = carry_b[at];
     carry_b[at] = S;          // what the chunk starts from
     S = fmaf(A, S, B);
@@ -355,7 +357,7 @@ __global__ __launch_bounds__(256) void rglru_chunk_apply_kernel(LruArgs a, const
   if (first >= end) return;
   const T* proj = (const T*)a.proj;
   T* out = (T*)a.out;
-  float S = carry_b[size_t(blockIdx.x) * a.width + c];
+  float S = carry_b[size_t(a.q_start[s] / kScanChunk + s + ci) * a.width + c];
   int t = first;
   for (; t + 8 <= end; t += 8) {
     float d[8], g[8], y[8];
@@ -476,7 +478,9 @@ __global__ __launch_bounds__(256) void retention_kernel(RetentionArgs a) {
 // Only powers of g with exponents >= 0 appear (nothing is divided by a power), so a small decay loses nothing.
 // First every chunk's own sum U = sum_j g^(n-1-j) k_j v_j^T; then per state element the chunks one after the other, which
 // leaves in U's place the state each chunk starts from; then every chunk's outputs.  scratch: float32
-// [requests * chunks, heads, dim, vdim].  A thread block is 8 rows of 32 threads.
+// [T / C + requests, heads, dim, vdim]: chunk ci of request s has row q_start[s] / C + s + ci, which keeps the requests'
+// rows apart (a request of n tokens has at most n / C + 1 chunks) however unequal their portions are.  A thread block is 8
+// rows of 32 threads.
 template <typename T>
 __device__ __forceinline__ float turned(const T* src, const float* cos_sin, size_t t, int d, int half) {
   if (d < 2 * half) {
@@ -558,7 +562,7 @@ __global__ __launch_bounds__(256) void retention_chunk_local_kernel(RetentionArg
   }
   __syncthreads();
   const int tx = threadIdx.x % 32, ty = threadIdx.x / 32;
-  float* U = scratch + (size_t(blockIdx.x) * a.heads + h) * D * V;
+  float* U = scratch + (size_t(a.q_start[s] / C + s + ci) * a.heads + h) * D * V;
   for (int d0 = 0; d0 < D; d0 += 32) {
     float acc[4][CV];
 #pragma unroll
@@ -602,7 +606,7 @@ __global__ __launch_bounds__(256) void retention_chunk_carry_kernel(RetentionArg
   float* kept = a.state + (size_t(slot) * a.heads + h) * DV + e;
   float S = *kept;
   const size_t step = size_t(a.heads) * DV;
-  float* at = scratch + (size_t(s) * chunks * a.heads + h) * DV + e;
+  float* at = scratch + (size_t(a.q_start[s] / C + s) * a.heads + h) * DV + e;
   const float whole = powf(gamma, float(C));
   int ci = 0;
   for (; ci + 8 <= used && (ci + 8) * C <= n; ci += 8, at += 8 * step) {      // eight whole chunks: their sums are asked for together
@@ -691,7 +695,7 @@ __global__ __launch_bounds__(256) void retention_chunk_apply_kernel(RetentionArg
   for (int r = 0; r < RPT; ++r)
 #pragma unroll
     for (int c = 0; c < CV; ++c) o[r][c] = 0.f;
-  const float* S0 = scratch + (size_t(blockIdx.x) * a.heads + h) * D * V;
+  const float* S0 = scratch + (size_t(a.q_start[s] / C + s + ci) * a.heads + h) * D * V;
   for (int d = 0; d < D; ++d) {      // what the tokens before the chunk left
     float qq[RPT], ss[CV];
 #pragma unroll
@@ -798,9 +802,9 @@ using namespace sprout;
 
 // float32 numbers of the scratch that a step whose longest portion has max_q_len tokens needs for its scan in chunks
 // (0: the scan walks each request in one go and needs none).
-extern "C" long long sp_rglru_carry_floats(int width, int n_seqs, int max_q_len) {
+extern "C" long long sp_rglru_carry_floats(int width, int n_seqs, int max_q_len, int T) {
   if (max_q_len <= 2 * kScanChunk) return 0;
-  return 2LL * n_seqs * ((max_q_len + kScanChunk - 1) / kScanChunk) * width;
+  return 2LL * (T / kScanChunk + n_seqs) * width;
 }
 
 extern "C" int sp_rglru_takes(int width, int blocks, int taps) {
@@ -859,7 +863,7 @@ extern "C" int sp_rglru(void* stream, int dtype, const void* proj, long long str
     const int chunks = (max_q_len + kScanChunk - 1) / kScanChunk;
     SP_REQUIRE((long long)n_seqs * chunks < (1 << 30), "sp_rglru: too many chunks");
     float* carry_a = carry;
-    float* carry_b = carry + size_t(n_seqs) * chunks * width;
+    float* carry_b = carry + size_t(T / kScanChunk + n_seqs) * width;
     const dim3 chunk_grid(n_seqs * chunks, scan_grid.y);
     rglru_chunk_local_kernel<<<chunk_grid, scan_threads, 0, s>>>(a, carry_a, carry_b, chunks);
     if (dtype == kF32) {
@@ -889,11 +893,11 @@ extern "C" int sp_retention_takes(int dim, int vdim) {
 
 // float32 numbers of the scratch that a step whose longest portion has max_q_len tokens needs for its walk in chunks
 // (0: every request's tokens are walked one after the other and none is needed).
-extern "C" long long sp_retention_scratch_floats(int heads, int dim, int vdim, int n_seqs, int max_q_len) {
+extern "C" long long sp_retention_scratch_floats(int heads, int dim, int vdim, int n_seqs, int max_q_len, int T) {
   if (max_q_len <= kRetentionLongPortion || heads <= 0 || dim <= 0 || vdim <= 0 || vdim > 256) return 0;
   const int C = retention_chunk_tokens(dim, vdim);
   if (C == 0) return 0;
-  return (long long)n_seqs * ((max_q_len + C - 1) / C) * heads * dim * vdim;
+  return ((long long)T / C + n_seqs) * heads * dim * vdim;
 }
 
 extern "C" int sp_retention(void* stream, int dtype, const void* proj, long long stride, int q_off, int k_off, int v_off, int g_off,
@@ -913,7 +917,7 @@ extern "C" int sp_retention(void* stream, int dtype, const void* proj, long long
   const int groups = vdim <= 256 ? 256 / vdim : 1, rows = (dim + groups - 1) / groups;
   RetentionArgs a = {proj, stride, q_off, k_off, v_off, g_off, heads, dim, vdim, rotary_dim, cos_sin, decay, eps, q_start, q_len,
                      state_slots, state, out, groups};
-  if (scratch && sp_retention_scratch_floats(heads, dim, vdim, n_seqs, max_q_len) > 0) {      // a long portion: its chunks side by side
+  if (scratch && sp_retention_scratch_floats(heads, dim, vdim, n_seqs, max_q_len, T) > 0) {      // a long portion: its chunks side by side
     if (dtype == kF32) return launch_retention_chunks<float>((hipStream_t)stream, a, n_seqs, max_q_len, scratch);
     return launch_retention_chunks<bf16_t>((hipStream_t)stream, a, n_seqs, max_q_len, scratch);
   }

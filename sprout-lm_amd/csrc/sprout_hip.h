@@ -278,7 +278,7 @@ int sp_rglru(void* stream, int dtype, const void* proj, long long stride, int y_
              int max_q_len, float* carry);
 // max_q_len: the most tokens one request brings to the step; carry: float32 scratch of sp_rglru_carry_floats numbers (null
 // or a short longest portion: every request's tokens are walked in one go, else in chunks side by side).
-long long sp_rglru_carry_floats(int width, int n_seqs, int max_q_len);
+long long sp_rglru_carry_floats(int width, int n_seqs, int max_q_len, int T);
 
 // Retention: per head S <- decay[h] S + k v^T, o = S^T q, with q and k turned by the angles of cos_sin ([T, rotary_dim / 2, 2]
 // of sp_rope_table: the first rotary_dim numbers of a head, d with d + rotary_dim / 2) and k times dim^(-1/2); o is divided
@@ -290,5 +290,5 @@ int sp_retention(void* stream, int dtype, const void* proj, long long stride, in
                  const int32_t* q_len, const int32_t* state_slots, float* state, void* out, int T, int n_seqs, int max_q_len,
                  float* scratch);
 // max_q_len, scratch: as for sp_rglru, with sp_retention_scratch_floats numbers.
-long long sp_retention_scratch_floats(int heads, int dim, int vdim, int n_seqs, int max_q_len);
+long long sp_retention_scratch_floats(int heads, int dim, int vdim, int n_seqs, int max_q_len, int T);
 }

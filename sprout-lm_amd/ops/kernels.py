@@ -795,7 +795,7 @@ def rglru(proj: torch.Tensor, y_off: int, x_off: int, width: int, blocks: int, t
         if t.dtype != torch.float32 or t.numel() < T * width:
             raise KernelError("rglru: scratch must hold float32 [T, width]")
     carry = None
-    need = library().sp_rglru_carry_floats(width, n_seqs, int(max_q_len)) if workspace is not None else 0
+    need = library().sp_rglru_carry_floats(width, n_seqs, int(max_q_len), T) if workspace is not None else 0
     if need:
         carry = workspace(need)
         if carry.dtype != torch.float32 or carry.numel() < need or not carry.is_cuda:
@@ -833,7 +833,7 @@ def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int
     for t, what in ((q_start, "q_start"), (q_len, "q_len"), (state_slots, "state_slots")):
         _ints(t, n_seqs, what)
     scratch = None
-    need = library().sp_retention_scratch_floats(heads, dim, vdim, n_seqs, int(max_q_len)) if workspace is not None else 0
+    need = library().sp_retention_scratch_floats(heads, dim, vdim, n_seqs, int(max_q_len), T) if workspace is not None else 0
     if need:
         scratch = workspace(need)
         if scratch.dtype != torch.float32 or scratch.numel() < need or not scratch.is_cuda:

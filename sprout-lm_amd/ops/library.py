@@ -85,9 +85,9 @@ def _declare(lib):
     }
     lib.sp_attention_workspace_floats.argtypes = [c_int] * 10
     lib.sp_attention_workspace_floats.restype = c_i64
-    lib.sp_rglru_carry_floats.argtypes = [c_int] * 3
+    lib.sp_rglru_carry_floats.argtypes = [c_int] * 4
     lib.sp_rglru_carry_floats.restype = c_i64
-    lib.sp_retention_scratch_floats.argtypes = [c_int] * 5
+    lib.sp_retention_scratch_floats.argtypes = [c_int] * 6
     lib.sp_retention_scratch_floats.restype = c_i64
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
