@@ -5,6 +5,7 @@
 // state_slots (one entry per request of the step) say where a request's tokens are and which row of the state tensors
 // is its own.  A kernel reads the state as the step before left it and leaves it for the next one.
 #include "common.h"
+#include "mfma.h"
 #include "sprout_hip.h"
 
 namespace sprout {
@@ -750,6 +751,329 @@ __global__ __launch_bounds__(256) void retention_chunk_apply_kernel(RetentionArg
   }
 }
 
+// Rows of q or k of a chunk into LDS [C][DP], turned, times `scale` and (where given) a weight per row; rows from `len` on
+// are zeros.  An item is a pair that turns together (one cosine and sine for both numbers) or a number that does not turn;
+// a thread's items are independent, so their loads are asked for together.
+template <typename T>
+__device__ __forceinline__ void load_turned_rows(float* dst, int DP, const T* rows, long long stride, const float* cos_sin,
+                                                 int first, int len, int C, int D, int half, float scale,
+                                                 const float* row_weight) {
+  // every load has an address that is valid whatever the item (rows past the end read the last row, and the result is dropped):
+  // loads under a condition would each wait on their own
+  const int W = D - half;
+  if (half > 0) {
+#pragma unroll 4
+    for (int e = threadIdx.x; e < C * W; e += blockDim.x) {
+      const int j = e / W, i = e % W, jj = min(j, len - 1);
+      const bool turns = i < half;
+      const T* src = rows + size_t(jj) * stride;
+      const float2 cs = reinterpret_cast<const float2*>(cos_sin)[size_t(first + jj) * half + (turns ? i : 0)];
+      const float x = to_float(src[turns ? i : i + half]), y = to_float(src[i + half]);
+      const float w = j < len ? (row_weight ? scale * row_weight[jj] : scale) : 0.f;
+      float* row = dst + j * DP;
+      if (turns) row[i] = (x * cs.x - y * cs.y) * w;
+      row[i + half] = turns ? (y * cs.x + x * cs.y) * w : y * w;
+    }
+  } else {
+#pragma unroll 4
+    for (int e = threadIdx.x; e < C * D; e += blockDim.x) {
+      const int j = e / D, i = e % D, jj = min(j, len - 1);
+      const float y = to_float(rows[size_t(jj) * stride + i]);
+      dst[j * DP + i] = j < len ? y * (row_weight ? scale * row_weight[jj] : scale) : 0.f;
+    }
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void load_value_rows(float* dst, const T* rows, long long stride, int len, int C, int V) {
+#pragma unroll 4
+  for (int e = threadIdx.x; e < C * V; e += blockDim.x) {
+    const int j = e / V, v = e % V;
+    const float value = to_float(rows[size_t(min(j, len - 1)) * stride + v]);
+    dst[e] = j < len ? value : 0.f;
+  }
+}
+
+// The chunk's rows in one go, for bfloat16 rows whose sizes and offsets are all in eights (16-byte loads) and small enough
+// that a thread has at most one group of eight of q, one of k and four of v: every load of a thread is asked for before
+// the first is used, so a block waits for memory once.  q_dst may be null (only k and v are wanted).
+__device__ __forceinline__ void unpack8(const uint4& p, float* f) {
+  const uint32_t w[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    f[2 * q] = __uint_as_float(w[q] << 16);
+    f[2 * q + 1] = __uint_as_float(w[q] & 0xffff0000u);
+  }
+}
+
+__device__ __forceinline__ void load_chunk_wide(const RetentionArgs& a, int h, int first, int len, int C, float* q_dst, float* k_dst,
+                                                float* v_dst, float k_scale, const float* k_weight) {
+  const int D = a.dim, V = a.vdim, half = a.rotary_dim / 2, DP = D + 1;
+  const bf16_t* proj = (const bf16_t*)a.proj;
+  const int groups = (D - half) / 8, items = C * groups, turning = half / 8;
+  const int tid = threadIdx.x, j = min(tid / groups, C - 1), g = tid % groups, jj = min(j, len - 1);
+  const bool turns = g < turning;
+  const int lo_at = turns ? 8 * g : 2 * half + 8 * (g - turning), hi_at = turns ? lo_at + half : lo_at;
+  const bf16_t* row = proj + size_t(first + jj) * a.stride;
+  const uint4 kx = ldg128(row + a.k_off + h * D + lo_at), ky = ldg128(row + a.k_off + h * D + hi_at);
+  uint4 qx = kx, qy = ky;
+  if (q_dst) {
+    qx = ldg128(row + a.q_off + h * D + lo_at);
+    qy = ldg128(row + a.q_off + h * D + hi_at);
+  }
+  float4 cs[4] = {};
+  if (half > 0) {
+    const float4* at = reinterpret_cast<const float4*>(a.cos_sin + (size_t(first + jj) * half + (turns ? 8 * g : 0)) * 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) cs[i] = at[i];
+  }
+  const int v_groups = V / 8, v_items = C * v_groups;
+  uint4 vv[4];
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int e = min(tid + 256 * it, v_items - 1), vj = min(e / v_groups, len - 1);
+    vv[it] = ldg128(proj + size_t(first + vj) * a.stride + a.v_off + h * V + 8 * (e % v_groups));
+  }
+  if (tid < items) {
+    const bool in = j < len;
+    const float wk = in ? (k_weight ? k_scale * k_weight[jj] : k_scale) : 0.f, wq = in ? 1.f : 0.f;
+    float x[8], y[8];
+    const float c[16] = {cs[0].x, cs[0].y, cs[0].z, cs[0].w, cs[1].x, cs[1].y, cs[1].z, cs[1].w,
+                         cs[2].x, cs[2].y, cs[2].z, cs[2].w, cs[3].x, cs[3].y, cs[3].z, cs[3].w};
+    unpack8(kx, x);
+    unpack8(ky, y);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (turns) {
+        k_dst[j * DP + lo_at + i] = (x[i] * c[2 * i] - y[i] * c[2 * i + 1]) * wk;
+        k_dst[j * DP + hi_at + i] = (y[i] * c[2 * i] + x[i] * c[2 * i + 1]) * wk;
+      } else {
+        k_dst[j * DP + lo_at + i] = x[i] * wk;
+      }
+    }
+    if (q_dst) {
+      unpack8(qx, x);
+      unpack8(qy, y);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (turns) {
+          q_dst[j * DP + lo_at + i] = (x[i] * c[2 * i] - y[i] * c[2 * i + 1]) * wq;
+          q_dst[j * DP + hi_at + i] = (y[i] * c[2 * i] + x[i] * c[2 * i + 1]) * wq;
+        } else {
+          q_dst[j * DP + lo_at + i] = x[i] * wq;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    const int e = tid + 256 * it;
+    if (e >= v_items) break;
+    float f[8];
+    unpack8(vv[it], f);
+    const int vj = e / v_groups;
+    float* dst = v_dst + vj * V + 8 * (e % v_groups);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) dst[i] = vj < len ? f[i] : 0.f;
+  }
+}
+
+// Whether load_chunk_wide takes the rows (decided on the host).
+static bool retention_wide_rows(int dtype, const RetentionArgs& a, int C) {
+  const int half = a.rotary_dim / 2;
+  const bool eights = a.dim % 8 == 0 && half % 8 == 0 && a.vdim % 8 == 0 && a.stride % 8 == 0 && a.q_off % 8 == 0 && a.k_off % 8 == 0 &&
+                      a.v_off % 8 == 0;
+  return dtype == kBF16 && eights && a.dim > half && C * ((a.dim - half) / 8) <= 256 && C * (a.vdim / 8) <= 1024 &&
+         (reinterpret_cast<uintptr_t>(a.proj) % 16) == 0 && (reinterpret_cast<uintptr_t>(a.cos_sin) % 16) == 0;
+}
+
+// The same three passes with the products on the matrix cores' float32 instruction (32x32x2: float32 operands and sums, no
+// reduced precision), chunks of 32 tokens, a block of four waves per (chunk, head).  Lane l of a wave gives the instruction
+// A[l % 32][l / 32] and B[l / 32][l % 32] and holds D[8 (r / 4) + 4 (l / 32) + r % 4][l % 32] in element r.
+constexpr int kMfmaChunk = 32;
+
+// U [dim][vdim] = sum_j (g^(n-1-j) k_j) v_j^T: a wave a tile of 32 x 32, the chunk's tokens two at a time.
+template <typename T>
+__global__ __launch_bounds__(256) void retention_mfma_local_kernel(RetentionArgs a, float* __restrict__ scratch, int chunks, int wide) {
+  extern __shared__ float lds[];      // k [C][D + 1] (times its power of the decay), v [C][V]; rows past the chunk's end are zeros
+  constexpr int C = kMfmaChunk;
+  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, h = blockIdx.y;
+  const int D = a.dim, V = a.vdim, half = a.rotary_dim / 2, DP = D + 1;
+  const int first = a.q_start[s] + ci * C, len = min(C, a.q_start[s] + a.q_len[s] - first);
+  if (len <= 0) return;
+  float* ks = lds;
+  float* vs = lds + C * DP;
+  __shared__ float weight[C];      // g^(n-1-j)
+  const float gamma = a.decay[h], k_scale = 1.0f / sqrtf(float(D));
+  const T* proj = (const T*)a.proj;
+  if (threadIdx.x < C) weight[threadIdx.x] = threadIdx.x < len ? powf(gamma, float(len - 1 - threadIdx.x)) : 0.f;
+  if (!wide) load_value_rows(vs, proj + size_t(first) * a.stride + a.v_off + h * V, a.stride, len, C, V);
+  __syncthreads();
+  if (wide) load_chunk_wide(a, h, first, len, C, nullptr, ks, vs, k_scale, weight);
+  else load_turned_rows(ks, DP, proj + size_t(first) * a.stride + a.k_off + h * D, a.stride, a.cos_sin, first, len, C, D, half, k_scale,
+                        weight);
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, hi = lane >> 5;
+  const int tiles_v = (V + 31) / 32, tiles = ((D + 31) / 32) * tiles_v;
+  float* U = scratch + (size_t(a.q_start[s] / C + s + ci) * a.heads + h) * D * V;
+  for (int tile = wave; tile < tiles; tile += 4) {
+    const int d0 = (tile / tiles_v) * 32, v0 = (tile % tiles_v) * 32, d = d0 + col, v = v0 + col;
+    floatx16 acc = {0};
+#pragma unroll
+    for (int kk = 0; kk < C / 2; ++kk) {
+      const int j = 2 * kk + hi;
+      acc = mfma32_f32(d < D ? ks[j * DP + d] : 0.f, v < V ? vs[j * V + v] : 0.f, acc);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = d0 + 8 * (r / 4) + 4 * hi + r % 4;
+      if (row < D && v < V) U[size_t(row) * V + v] = acc[r];
+    }
+  }
+}
+
+// The chunk's outputs.  Scores: the four waves share the key dimension and wave 0 sums, masks and weighs them; then a wave a
+// tile of 32 value columns (NT tiles a wave): g^(i+1) q_i S0 over dim, the weighted scores times the values over the chunk's
+// tokens, in one accumulator; the heads' unit norm over all columns through LDS; the gate; the store.
+template <typename T, int NT>
+__global__ __launch_bounds__(256) void retention_mfma_apply_kernel(RetentionArgs a, const float* __restrict__ scratch, int chunks, int wide) {
+  extern __shared__ float lds[];      // q, k [C][D + 1], v [C][V], weights [C][C + 1], powers [C + 1], three partial score tiles, row sums [4][C]
+  constexpr int C = kMfmaChunk, CP = C + 1;
+  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, h = blockIdx.y;
+  const int D = a.dim, V = a.vdim, half = a.rotary_dim / 2, DP = D + 1;
+  const int first = a.q_start[s] + ci * C, len = min(C, a.q_start[s] + a.q_len[s] - first);
+  if (len <= 0) return;
+  float* qs = lds;
+  float* ks = qs + C * DP;
+  float* vs = ks + C * DP;
+  float* ps = vs + C * V;
+  float* pw = ps + C * CP;
+  float* parts = pw + CP;             // [3][C][CP]
+  float* squares = parts + 3 * C * CP;   // [4][C]
+  const float gamma = a.decay[h], k_scale = 1.0f / sqrtf(float(D));
+  const T* proj = (const T*)a.proj;
+  T* out = (T*)a.out;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, col = lane & 31, hi = lane >> 5;
+  const float* S0 = scratch + (size_t(a.q_start[s] / C + s + ci) * a.heads + h) * D * V;
+  // what the wave's first tile needs from memory later is asked for now, with the chunk's rows: the state before the chunk
+  // (its first 2 PRE rows) and the gates; addresses are valid whatever the lane, what is not needed is dropped
+  constexpr int PRE = 32;
+  float kept0[PRE], gate0[16];
+  {
+    const int vc = min(wave * 32 + col, V - 1);
+#pragma unroll
+    for (int kk = 0; kk < PRE; ++kk) kept0[kk] = S0[size_t(min(2 * kk + hi, D - 1)) * V + vc];
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      gate0[r] = to_float(proj[size_t(first + min(8 * (r / 4) + 4 * hi + r % 4, len - 1)) * a.stride + a.g_off + h * V + vc]);
+  }
+  if (wide) {
+    load_chunk_wide(a, h, first, len, C, qs, ks, vs, k_scale, nullptr);
+  } else {
+    load_turned_rows(qs, DP, proj + size_t(first) * a.stride + a.q_off + h * D, a.stride, a.cos_sin, first, len, C, D, half, 1.0f,
+                     (const float*)nullptr);
+    load_turned_rows(ks, DP, proj + size_t(first) * a.stride + a.k_off + h * D, a.stride, a.cos_sin, first, len, C, D, half, k_scale,
+                     (const float*)nullptr);
+    load_value_rows(vs, proj + size_t(first) * a.stride + a.v_off + h * V, a.stride, len, C, V);
+  }
+  for (int e = threadIdx.x; e <= C; e += blockDim.x) pw[e] = powf(gamma, float(e));
+  __syncthreads();
+  {
+    const int steps = (D + 1) / 2, share = (steps + 3) / 4, kk_end = min(steps, (wave + 1) * share);
+    floatx16 acc = {0};
+    for (int kk = wave * share; kk < kk_end; ++kk) {
+      const int d = 2 * kk + hi;
+      const bool in = d < D;
+      acc = mfma32_f32(in ? qs[col * DP + d] : 0.f, in ? ks[col * DP + d] : 0.f, acc);
+    }
+    if (wave) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) parts[((wave - 1) * C + 8 * (r / 4) + 4 * hi + r % 4) * CP + col] = acc[r];
+    }
+    __syncthreads();
+    if (wave == 0) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int i = 8 * (r / 4) + 4 * hi + r % 4, j = col;
+        const float sum = ((acc[r] + parts[i * CP + j]) + parts[(C + i) * CP + j]) + parts[(2 * C + i) * CP + j];
+        ps[i * CP + j] = j <= i ? sum * pw[i - j] : 0.f;
+      }
+    }
+    __syncthreads();
+  }
+  const int tiles_v = (V + 31) / 32;
+  floatx16 o[NT];
+  float sq[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) sq[r] = 0.f;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    o[t] = floatx16{0};
+    const int tile = wave + 4 * t;
+    if (tile >= tiles_v) continue;
+    const int v = tile * 32 + col;
+    const bool live = v < V;
+    const float weight = pw[col + 1];
+    const int steps = (D + 1) / 2;
+    int kk0 = 0;
+    if (t == 0) {      // what the tokens before the chunk left: first from the rows asked for at the start
+#pragma unroll
+      for (int kk = 0; kk < PRE; ++kk) {
+        const int d = 2 * kk + hi;
+        const bool in = d < D;
+        if (kk < steps) o[t] = mfma32_f32(in ? qs[col * DP + d] * weight : 0.f, in && live ? kept0[kk] : 0.f, o[t]);
+      }
+      kk0 = PRE;
+    }
+#pragma unroll 8
+    for (int kk = kk0; kk < steps; ++kk) {
+      const int d = 2 * kk + hi;
+      const bool in = d < D;
+      const float kept = S0[size_t(min(d, D - 1)) * V + min(v, V - 1)];      // always a valid address: the loads do not wait on each other
+      o[t] = mfma32_f32(in ? qs[col * DP + d] * weight : 0.f, in && live ? kept : 0.f, o[t]);
+    }
+#pragma unroll
+    for (int kk = 0; kk < C / 2; ++kk) {      // the chunk's own tokens
+      const int j = 2 * kk + hi;
+      o[t] = mfma32_f32(ps[col * CP + j], live ? vs[j * V + v] : 0.f, o[t]);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sq[r] = fmaf(o[t][r], o[t][r], sq[r]);      // columns past V hold zeros
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float total = sq[r];
+#pragma unroll
+    for (int off = 16; off > 0; off >>= 1) total += __shfl_xor(total, off);
+    if (col == 0) squares[wave * C + 8 * (r / 4) + 4 * hi + r % 4] = total;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int tile = wave + 4 * t, v = tile * 32 + col;
+    if (tile >= tiles_v || v >= V) continue;
+    float g[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+      g[r] = t == 0 ? gate0[r]
+                    : to_float(proj[size_t(first + min(8 * (r / 4) + 4 * hi + r % 4, len - 1)) * a.stride + a.g_off + h * V + v]);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int i = 8 * (r / 4) + 4 * hi + r % 4;
+      if (i >= len) continue;
+      const float total = ((squares[i] + squares[C + i]) + squares[2 * C + i]) + squares[3 * C + i];
+      const float unit = 1.0f / sqrtf(total / float(V) + a.eps);
+      out[(size_t(first + i) * a.heads + h) * V + v] = from_float<T>((o[t][r] * unit) * (g[r] * sigmoid(g[r])));
+    }
+  }
+}
+
+static size_t retention_mfma_lds(int dim, int vdim) {
+  constexpr int C = kMfmaChunk;
+  return sizeof(float) * (size_t(2) * C * (dim + 1) + size_t(C) * vdim + size_t(4) * C * (C + 1) + (C + 1) + 4 * C);
+}
+static bool retention_mfma_fits(int dim, int vdim) { return vdim <= 256 && retention_mfma_lds(dim, vdim) <= 64 * 1024; }
+
 constexpr int kRetentionLongPortion = 8;      // a step whose longest portion has more tokens takes the chunks
 
 static size_t retention_chunk_lds(int C, int dim, int vdim) {
@@ -757,6 +1081,7 @@ static size_t retention_chunk_lds(int C, int dim, int vdim) {
 }
 // Tokens per chunk: the most whose tiles fit 64 KB of LDS (0: none do).
 static int retention_chunk_tokens(int dim, int vdim) {
+  if (retention_mfma_fits(dim, vdim)) return kMfmaChunk;      // the matrix cores' kernels
   for (int C : {64, 32, 16})
     if (retention_chunk_lds(C, dim, vdim) <= 64 * 1024) return C;
   return 0;
@@ -768,6 +1093,15 @@ static int launch_retention_chunks(hipStream_t s, const RetentionArgs& a, int n_
   SP_REQUIRE((long long)n_seqs * chunks < (1 << 30), "sp_retention: too many chunks");
   const dim3 grid(n_seqs * chunks, a.heads);
   const size_t local_lds = sizeof(float) * (size_t(C) * (a.dim + 1) + size_t(C) * a.vdim);
+  if (retention_mfma_fits(a.dim, a.vdim)) {
+    const int wide = retention_wide_rows(sizeof(T) == 2 ? kBF16 : kF32, a, C);
+    retention_mfma_local_kernel<T><<<grid, 256, local_lds, s>>>(a, scratch, chunks, wide);
+    retention_chunk_carry_kernel<<<dim3(n_seqs, a.heads, (DV + 255) / 256), 256, 0, s>>>(a, scratch, chunks, C);
+    const size_t mfma_lds = retention_mfma_lds(a.dim, a.vdim);
+    if (a.vdim <= 128) retention_mfma_apply_kernel<T, 1><<<grid, 256, mfma_lds, s>>>(a, scratch, chunks, wide);
+    else retention_mfma_apply_kernel<T, 2><<<grid, 256, mfma_lds, s>>>(a, scratch, chunks, wide);
+    return check_launch("sp_retention (chunks on the matrix cores)");
+  }
   retention_chunk_local_kernel<T, CV><<<grid, 256, local_lds, s>>>(a, scratch, chunks, C);
   retention_chunk_carry_kernel<<<dim3(n_seqs, a.heads, (DV + 255) / 256), 256, 0, s>>>(a, scratch, chunks, C);
   const size_t lds = retention_chunk_lds(C, a.dim, a.vdim);
