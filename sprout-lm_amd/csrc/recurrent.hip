@@ -16,6 +16,24 @@ __device__ __forceinline__ float gelu_tanh(float z) {
 __device__ __forceinline__ float softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 __device__ __forceinline__ float sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
 
+// Kernels that take a block per chunk number the chunks of a step's requests without gaps to speak of: chunk ci of request
+// r is number q_start[r] / C + r + ci (a request of n tokens has at most n / C + 1 chunks, so the numbers of two requests
+// never meet), and T / C + requests blocks cover them all, however unequal the requests' portions are.  Which request and
+// chunk a number means: the last request whose first number is not above it (the requests' few descriptors are the same for
+// the whole block).  False: the number is one of the few that no chunk has.
+__device__ __forceinline__ bool chunk_of_block(const int32_t* q_start, const int32_t* q_len, int n_seqs, int C, int number,
+                                               int& request, int& chunk) {
+  int lo = 0, hi = n_seqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (q_start[mid] / C + mid <= number) lo = mid;
+    else hi = mid - 1;
+  }
+  request = lo;
+  chunk = number - (q_start[lo] / C + lo);
+  return chunk * C < q_len[lo];
+}
+
 // ------------------------------------------------------------------------------------------------ gated linear recurrence
 struct LruArgs {
   const void* proj;            // [T, stride]: the gate branch (before its activation) at y_off, the recurrent branch at x_off
@@ -295,8 +313,10 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(LruArgs a) {
 constexpr int kScanChunk = 64;
 
 __global__ __launch_bounds__(256) void rglru_chunk_local_kernel(LruArgs a, float* __restrict__ carry_a,
-                                                                float* __restrict__ carry_b, int chunks) {
-  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, c = blockIdx.y * blockDim.x + threadIdx.x;
+                                                                float* __restrict__ carry_b, int n_seqs) {
+  int s, ci;
+  if (!chunk_of_block(a.q_start, a.q_len, n_seqs, kScanChunk, blockIdx.x, s, ci)) return;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= a.width) return;
   const int first = a.q_start[s] + ci * kScanChunk, end = min(first + kScanChunk, a.q_start[s] + a.q_len[s]);
   if (first >= end) return;
@@ -333,11 +353,22 @@ __global__ __launch_bounds__(256) void rglru_chunk_carry_kernel(LruArgs a, const
   const int start = a.q_start[s], n = a.q_len[s], slot = a.state_slots[s];
   const int used = (n + kScanChunk - 1) / kScanChunk;
   float S = a.state[size_t(slot) * a.width + c];
-  for (int ci = 0; ci < used; ++ci) {
-    const size_t at = (size_t(start / kScanChunk + s) + ci) * a.width + c;
-    const float A = carry_a[at], B = carry_b[at];
-    carry_b[at] = S;          // what the chunk starts from
-    S = fmaf(A, S, B);
+  const size_t base = size_t(start / kScanChunk + s) * a.width + c;
+  for (int ci = 0; ci < used; ci += 8) {      // eight chunks' products and sums are asked for together
+    float A[8], B[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const size_t at = base + size_t(min(ci + j, used - 1)) * a.width;
+      A[j] = carry_a[at];
+      B[j] = carry_b[at];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (ci + j < used) {
+        carry_b[base + size_t(ci + j) * a.width] = S;          // what the chunk starts from
+        S = fmaf(A[j], S, B[j]);
+      }
+    }
   }
   a.state[size_t(slot) * a.width + c] = S;
   const T* proj = (const T*)a.proj;
@@ -351,8 +382,10 @@ __global__ __launch_bounds__(256) void rglru_chunk_carry_kernel(LruArgs a, const
 }
 
 template <typename T>
-__global__ __launch_bounds__(256) void rglru_chunk_apply_kernel(LruArgs a, const float* __restrict__ carry_b, int chunks) {
-  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, c = blockIdx.y * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(256) void rglru_chunk_apply_kernel(LruArgs a, const float* __restrict__ carry_b, int n_seqs) {
+  int s, ci;
+  if (!chunk_of_block(a.q_start, a.q_len, n_seqs, kScanChunk, blockIdx.x, s, ci)) return;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= a.width) return;
   const int first = a.q_start[s] + ci * kScanChunk, end = min(first + kScanChunk, a.q_start[s] + a.q_len[s]);
   if (first >= end) return;
@@ -542,9 +575,11 @@ __global__ __launch_bounds__(256) void retention_general_kernel(RetentionArgs a)
 }
 
 template <typename T, int CV>
-__global__ __launch_bounds__(256) void retention_chunk_local_kernel(RetentionArgs a, float* __restrict__ scratch, int chunks, int C) {
+__global__ __launch_bounds__(256) void retention_chunk_local_kernel(RetentionArgs a, float* __restrict__ scratch, int n_seqs, int C) {
   extern __shared__ float lds[];      // k [C][D + 1] (times its power of the decay), v [C][V]
-  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, h = blockIdx.y;
+  int s, ci;
+  if (!chunk_of_block(a.q_start, a.q_len, n_seqs, C, blockIdx.x, s, ci)) return;
+  const int h = blockIdx.y;
   const int D = a.dim, V = a.vdim, half = a.rotary_dim / 2, DP = D + 1;
   const int first = a.q_start[s] + ci * C, len = min(C, a.q_start[s] + a.q_len[s] - first);
   if (len <= 0) return;
@@ -608,31 +643,29 @@ __global__ __launch_bounds__(256) void retention_chunk_carry_kernel(RetentionArg
   float S = *kept;
   const size_t step = size_t(a.heads) * DV;
   float* at = scratch + (size_t(a.q_start[s] / C + s) * a.heads + h) * DV + e;
-  const float whole = powf(gamma, float(C));
-  int ci = 0;
-  for (; ci + 8 <= used && (ci + 8) * C <= n; ci += 8, at += 8 * step) {      // eight whole chunks: their sums are asked for together
+  const float whole = powf(gamma, float(C)), last = powf(gamma, float(n - (used - 1) * C));
+  for (int ci = 0; ci < used; ci += 8) {      // eight chunks' sums are asked for together (past the last: the last one's again)
     float U[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) U[j] = at[j * step];
+    for (int j = 0; j < 8; ++j) U[j] = at[size_t(min(ci + j, used - 1)) * step];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      at[j * step] = S;          // what the chunk starts from
-      S = fmaf(whole, S, U[j]);
+      if (ci + j < used) {
+        at[size_t(ci + j) * step] = S;          // what the chunk starts from
+        S = fmaf(ci + j == used - 1 ? last : whole, S, U[j]);
+      }
     }
-  }
-  for (; ci < used; ++ci, at += step) {
-    const float U = *at;
-    *at = S;
-    S = fmaf(powf(gamma, float(min(C, n - ci * C))), S, U);
   }
   *kept = S;
 }
 
 template <typename T, int C, int CV>
-__global__ __launch_bounds__(256) void retention_chunk_apply_kernel(RetentionArgs a, const float* __restrict__ scratch, int chunks) {
+__global__ __launch_bounds__(256) void retention_chunk_apply_kernel(RetentionArgs a, const float* __restrict__ scratch, int n_seqs) {
   extern __shared__ float lds[];      // q, k [C][D + 1], v [C][V], weights [C][C + 1], powers of the decay [C + 1]
   constexpr int RPT = C / 8, JC = (C + 31) / 32, CP = C + 1;
-  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, h = blockIdx.y;
+  int s, ci;
+  if (!chunk_of_block(a.q_start, a.q_len, n_seqs, C, blockIdx.x, s, ci)) return;
+  const int h = blockIdx.y;
   const int D = a.dim, V = a.vdim, half = a.rotary_dim / 2, DP = D + 1;
   const int first = a.q_start[s] + ci * C, len = min(C, a.q_start[s] + a.q_len[s] - first);
   if (len <= 0) return;
@@ -894,10 +927,12 @@ constexpr int kMfmaChunk = 32;
 
 // U [dim][vdim] = sum_j (g^(n-1-j) k_j) v_j^T: a wave a tile of 32 x 32, the chunk's tokens two at a time.
 template <typename T>
-__global__ __launch_bounds__(256) void retention_mfma_local_kernel(RetentionArgs a, float* __restrict__ scratch, int chunks, int wide) {
+__global__ __launch_bounds__(256) void retention_mfma_local_kernel(RetentionArgs a, float* __restrict__ scratch, int n_seqs, int wide) {
   extern __shared__ float lds[];      // k [C][D + 1] (times its power of the decay), v [C][V]; rows past the chunk's end are zeros
   constexpr int C = kMfmaChunk;
-  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, h = blockIdx.y;
+  int s, ci;
+  if (!chunk_of_block(a.q_start, a.q_len, n_seqs, C, blockIdx.x, s, ci)) return;
+  const int h = blockIdx.y;
   const int D = a.dim, V = a.vdim, half = a.rotary_dim / 2, DP = D + 1;
   const int first = a.q_start[s] + ci * C, len = min(C, a.q_start[s] + a.q_len[s] - first);
   if (len <= 0) return;
@@ -936,10 +971,12 @@ __global__ __launch_bounds__(256) void retention_mfma_local_kernel(RetentionArgs
 // tile of 32 value columns (NT tiles a wave): g^(i+1) q_i S0 over dim, the weighted scores times the values over the chunk's
 // tokens, in one accumulator; the heads' unit norm over all columns through LDS; the gate; the store.
 template <typename T, int NT>
-__global__ __launch_bounds__(256) void retention_mfma_apply_kernel(RetentionArgs a, const float* __restrict__ scratch, int chunks, int wide) {
+__global__ __launch_bounds__(256) void retention_mfma_apply_kernel(RetentionArgs a, const float* __restrict__ scratch, int n_seqs, int wide) {
   extern __shared__ float lds[];      // q, k [C][D + 1], v [C][V], weights [C][C + 1], powers [C + 1], three partial score tiles, row sums [4][C]
   constexpr int C = kMfmaChunk, CP = C + 1;
-  const int s = blockIdx.x / chunks, ci = blockIdx.x % chunks, h = blockIdx.y;
+  int s, ci;
+  if (!chunk_of_block(a.q_start, a.q_len, n_seqs, C, blockIdx.x, s, ci)) return;
+  const int h = blockIdx.y;
   const int D = a.dim, V = a.vdim, half = a.rotary_dim / 2, DP = D + 1;
   const int first = a.q_start[s] + ci * C, len = min(C, a.q_start[s] + a.q_len[s] - first);
   if (len <= 0) return;
@@ -1088,36 +1125,36 @@ static int retention_chunk_tokens(int dim, int vdim) {
 }
 
 template <typename T, int CV>
-static int launch_retention_chunks(hipStream_t s, const RetentionArgs& a, int n_seqs, int max_q_len, float* scratch) {
+static int launch_retention_chunks(hipStream_t s, const RetentionArgs& a, int n_seqs, int max_q_len, int T_tokens, float* scratch) {
   const int C = retention_chunk_tokens(a.dim, a.vdim), chunks = (max_q_len + C - 1) / C, DV = a.dim * a.vdim;
   SP_REQUIRE((long long)n_seqs * chunks < (1 << 30), "sp_retention: too many chunks");
-  const dim3 grid(n_seqs * chunks, a.heads);
+  const dim3 grid(T_tokens / C + n_seqs, a.heads);      // a block per chunk number (chunk_of_block)
   const size_t local_lds = sizeof(float) * (size_t(C) * (a.dim + 1) + size_t(C) * a.vdim);
   if (retention_mfma_fits(a.dim, a.vdim)) {
     const int wide = retention_wide_rows(sizeof(T) == 2 ? kBF16 : kF32, a, C);
-    retention_mfma_local_kernel<T><<<grid, 256, local_lds, s>>>(a, scratch, chunks, wide);
+    retention_mfma_local_kernel<T><<<grid, 256, local_lds, s>>>(a, scratch, n_seqs, wide);
     retention_chunk_carry_kernel<<<dim3(n_seqs, a.heads, (DV + 255) / 256), 256, 0, s>>>(a, scratch, chunks, C);
     const size_t mfma_lds = retention_mfma_lds(a.dim, a.vdim);
-    if (a.vdim <= 128) retention_mfma_apply_kernel<T, 1><<<grid, 256, mfma_lds, s>>>(a, scratch, chunks, wide);
-    else retention_mfma_apply_kernel<T, 2><<<grid, 256, mfma_lds, s>>>(a, scratch, chunks, wide);
+    if (a.vdim <= 128) retention_mfma_apply_kernel<T, 1><<<grid, 256, mfma_lds, s>>>(a, scratch, n_seqs, wide);
+    else retention_mfma_apply_kernel<T, 2><<<grid, 256, mfma_lds, s>>>(a, scratch, n_seqs, wide);
     return check_launch("sp_retention (chunks on the matrix cores)");
   }
-  retention_chunk_local_kernel<T, CV><<<grid, 256, local_lds, s>>>(a, scratch, chunks, C);
+  retention_chunk_local_kernel<T, CV><<<grid, 256, local_lds, s>>>(a, scratch, n_seqs, C);
   retention_chunk_carry_kernel<<<dim3(n_seqs, a.heads, (DV + 255) / 256), 256, 0, s>>>(a, scratch, chunks, C);
   const size_t lds = retention_chunk_lds(C, a.dim, a.vdim);
-  if (C == 64) retention_chunk_apply_kernel<T, 64, CV><<<grid, 256, lds, s>>>(a, scratch, chunks);
-  else if (C == 32) retention_chunk_apply_kernel<T, 32, CV><<<grid, 256, lds, s>>>(a, scratch, chunks);
-  else retention_chunk_apply_kernel<T, 16, CV><<<grid, 256, lds, s>>>(a, scratch, chunks);
+  if (C == 64) retention_chunk_apply_kernel<T, 64, CV><<<grid, 256, lds, s>>>(a, scratch, n_seqs);
+  else if (C == 32) retention_chunk_apply_kernel<T, 32, CV><<<grid, 256, lds, s>>>(a, scratch, n_seqs);
+  else retention_chunk_apply_kernel<T, 16, CV><<<grid, 256, lds, s>>>(a, scratch, n_seqs);
   return check_launch("sp_retention (chunks)");
 }
 
 template <typename T>
-static int launch_retention_chunks(hipStream_t s, const RetentionArgs& a, int n_seqs, int max_q_len, float* scratch) {
+static int launch_retention_chunks(hipStream_t s, const RetentionArgs& a, int n_seqs, int max_q_len, int T_tokens, float* scratch) {
   const int cv = (a.vdim + 31) / 32;
-  if (cv <= 1) return launch_retention_chunks<T, 1>(s, a, n_seqs, max_q_len, scratch);
-  if (cv <= 2) return launch_retention_chunks<T, 2>(s, a, n_seqs, max_q_len, scratch);
-  if (cv <= 4) return launch_retention_chunks<T, 4>(s, a, n_seqs, max_q_len, scratch);
-  return launch_retention_chunks<T, 8>(s, a, n_seqs, max_q_len, scratch);
+  if (cv <= 1) return launch_retention_chunks<T, 1>(s, a, n_seqs, max_q_len, T_tokens, scratch);
+  if (cv <= 2) return launch_retention_chunks<T, 2>(s, a, n_seqs, max_q_len, T_tokens, scratch);
+  if (cv <= 4) return launch_retention_chunks<T, 4>(s, a, n_seqs, max_q_len, T_tokens, scratch);
+  return launch_retention_chunks<T, 8>(s, a, n_seqs, max_q_len, T_tokens, scratch);
 }
 
 template <typename T>
@@ -1198,14 +1235,14 @@ extern "C" int sp_rglru(void* stream, int dtype, const void* proj, long long str
     SP_REQUIRE((long long)n_seqs * chunks < (1 << 30), "sp_rglru: too many chunks");
     float* carry_a = carry;
     float* carry_b = carry + size_t(T / kScanChunk + n_seqs) * width;
-    const dim3 chunk_grid(n_seqs * chunks, scan_grid.y);
-    rglru_chunk_local_kernel<<<chunk_grid, scan_threads, 0, s>>>(a, carry_a, carry_b, chunks);
+    const dim3 chunk_grid(T / kScanChunk + n_seqs, scan_grid.y);      // a block per chunk number (chunk_of_block)
+    rglru_chunk_local_kernel<<<chunk_grid, scan_threads, 0, s>>>(a, carry_a, carry_b, n_seqs);
     if (dtype == kF32) {
       rglru_chunk_carry_kernel<float><<<scan_grid, scan_threads, 0, s>>>(a, carry_a, carry_b, chunks);
-      rglru_chunk_apply_kernel<float><<<chunk_grid, scan_threads, 0, s>>>(a, carry_b, chunks);
+      rglru_chunk_apply_kernel<float><<<chunk_grid, scan_threads, 0, s>>>(a, carry_b, n_seqs);
     } else {
       rglru_chunk_carry_kernel<bf16_t><<<scan_grid, scan_threads, 0, s>>>(a, carry_a, carry_b, chunks);
-      rglru_chunk_apply_kernel<bf16_t><<<chunk_grid, scan_threads, 0, s>>>(a, carry_b, chunks);
+      rglru_chunk_apply_kernel<bf16_t><<<chunk_grid, scan_threads, 0, s>>>(a, carry_b, n_seqs);
     }
     return check_launch("sp_rglru (scan in chunks)");
   }
@@ -1252,8 +1289,8 @@ extern "C" int sp_retention(void* stream, int dtype, const void* proj, long long
   RetentionArgs a = {proj, stride, q_off, k_off, v_off, g_off, heads, dim, vdim, rotary_dim, cos_sin, decay, eps, q_start, q_len,
                      state_slots, state, out, groups};
   if (scratch && sp_retention_scratch_floats(heads, dim, vdim, n_seqs, max_q_len, T) > 0) {      // a long portion: its chunks side by side
-    if (dtype == kF32) return launch_retention_chunks<float>((hipStream_t)stream, a, n_seqs, max_q_len, scratch);
-    return launch_retention_chunks<bf16_t>((hipStream_t)stream, a, n_seqs, max_q_len, scratch);
+    if (dtype == kF32) return launch_retention_chunks<float>((hipStream_t)stream, a, n_seqs, max_q_len, T, scratch);
+    return launch_retention_chunks<bf16_t>((hipStream_t)stream, a, n_seqs, max_q_len, T, scratch);
   }
   if (!retention_in_registers(dim, vdim)) {
     const size_t general_lds = size_t(2 * dim + vdim) * sizeof(float);
