@@ -59,11 +59,11 @@ struct LruArgs {
   int T;
 };
 
-// The convolution outputs of TT tokens from t0 on, channels c0 .. c0 + n - 1, into u_s [TT][n].  Where a token lies in its
+// The convolution outputs of TT tokens from t0 on, channels c0 .. c0 + n - 1, into u_s [TT][ld].  Where a token lies in its
 // request's share of the step and which state row is its request's is looked up once per token, not once per channel, so
 // that the channels' loads do not each wait behind that chain.
 template <typename T, int TT>
-__device__ __forceinline__ void conv_outputs(const LruArgs& a, float* u_s, int t0, int c0, int n) {
+__device__ __forceinline__ void conv_outputs(const LruArgs& a, float* u_s, int t0, int c0, int n, int ld) {
   __shared__ int place[TT], row[TT];
   if (threadIdx.x < TT) {
     const int t = t0 + threadIdx.x;
@@ -85,16 +85,30 @@ __device__ __forceinline__ void conv_outputs(const LruArgs& a, float* u_s, int t
     float u = 0.f;
     if (t < a.T) {
       const int j = place[tt];
-      const float* tail = a.tail + size_t(row[tt]) * keep * a.width;
       u = to_float(((const T*)a.conv_b)[c]);
-      for (int tap = 0; tap < a.taps; ++tap) {
-        const int back = keep - tap;
-        const float x = j - back >= 0 ? to_float(proj[size_t(t - back) * a.stride + a.x_off + c])
-                                      : tail[size_t(keep + j - back) * a.width + c];
-        u = fmaf(to_float(((const T*)a.conv_w)[size_t(c) * a.taps + tap]), x, u);
+      if (j >= keep) {      // every tap's input is a token of this step: loads at addresses that are valid whatever the tap, so
+        // that they are asked for together (under a condition each would wait on its own), the sum in the taps' order
+#pragma unroll
+        for (int tap = 0; tap < 8; ++tap) {
+          const int tp = min(tap, keep);
+          const float w = to_float(((const T*)a.conv_w)[size_t(c) * a.taps + tp]);
+          const float x = to_float(proj[size_t(t - (keep - tp)) * a.stride + a.x_off + c]);
+          if (tap < a.taps) u = fmaf(w, x, u);
+        }
+        for (int tap = 8; tap < a.taps; ++tap)
+          u = fmaf(to_float(((const T*)a.conv_w)[size_t(c) * a.taps + tap]),
+                   to_float(proj[size_t(t - (keep - tap)) * a.stride + a.x_off + c]), u);
+      } else {
+        const float* tail = a.tail + size_t(row[tt]) * keep * a.width;
+        for (int tap = 0; tap < a.taps; ++tap) {
+          const int back = keep - tap;
+          const float x = j - back >= 0 ? to_float(proj[size_t(t - back) * a.stride + a.x_off + c])
+                                        : tail[size_t(keep + j - back) * a.width + c];
+          u = fmaf(to_float(((const T*)a.conv_w)[size_t(c) * a.taps + tap]), x, u);
+        }
       }
     }
-    u_s[e] = u;
+    u_s[tt * ld + e % n] = u;
   }
   __syncthreads();
 }
@@ -108,7 +122,7 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(LruArgs a, int lanes) 
   const int n = a.width / a.blocks, b = blockIdx.y, t0 = blockIdx.x * TT, c0 = b * n;
   const int slices = blockDim.x / lanes, lane = threadIdx.x % lanes, slice = threadIdx.x / lanes;
   float* sums = u_s + TT * n;
-  conv_outputs<T, TT>(a, u_s, t0, c0, n);
+  conv_outputs<T, TT>(a, u_s, t0, c0, n, n);
   const int share = (n + slices - 1) / slices, k_first = slice * share, k_end = min(n, k_first + share);
   for (int o0 = 0; o0 < n; o0 += lanes) {
     const int o = o0 + lane;
@@ -208,7 +222,7 @@ __global__ __launch_bounds__(256) void rglru_gates_few_kernel(LruArgs a, int sli
   const float bias_a0 = ends ? to_float(((const T*)a.ba)[c0 + o_first]) : 0.f;
   const float bias_i0 = ends ? to_float(((const T*)a.bi)[c0 + o_first]) : 0.f;
   const float lam0 = ends ? to_float(((const T*)a.lam)[c0 + o_first]) : 0.f;
-  conv_outputs<T, TT>(a, u_s, t0, c0, n);
+  conv_outputs<T, TT>(a, u_s, t0, c0, n, n);
   if (slice < slices) {
     float ra[TT][8], ri[TT][8];
 #pragma unroll
