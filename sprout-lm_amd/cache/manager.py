@@ -228,7 +228,9 @@ class CacheManager:
     @staticmethod
     def _first_needed(group, length: int) -> int:
         """The oldest key that the token at position `length` reads in `group`."""
-        return 0 if group.spec.window is None else max(0, length - group.spec.window + 1)
+        if group.spec.window is None or group.spec.keep_first > 0:      # kept first keys: read from the very first page on
+            return 0
+        return max(0, length - group.spec.window + 1)
 
     def publish(self, tokens, seq: SequenceCache, length: int | None = None) -> None:
         """Offer the full page of `seq` that ends at `length` (default: its computed length) for reuse.
@@ -344,8 +346,9 @@ class CacheManager:
         for gi, (g, blocks) in enumerate(zip(self.groups, seq.blocks)):
             if g.spec.window is None:
                 continue
-            # the next token (position new_length) reads keys >= new_length - window + 1
-            for i in range(self._first_needed(g, new_length) // g.page_tokens):
+            # the next token (position new_length) reads keys >= new_length - window + 1, and the first keep_first keys
+            kept_pages = -(-g.spec.keep_first // g.page_tokens)
+            for i in range(kept_pages, max(0, new_length - g.spec.window + 1) // g.page_tokens):
                 if blocks[i] != FREED:
                     g.pool.release(blocks[i])
                     blocks[i] = FREED

@@ -11,7 +11,9 @@ class PagedKVSpec:
     manager's size, which stays the unit in which prefixes are shared).
     value_dim None: values as wide as keys; else the width of a cached value where it differs from a key's
     `head_dim` (a mixer that caches a narrow rotated part beside a wide latent, say).
-    dtype None: the model's cache dtype; else the name of the dtype this slot is always kept in."""
+    dtype None: the model's cache dtype; else the name of the dtype this slot is always kept in.
+    keep_first: with a window, a request's first `keep_first` keys stay readable as long as it lives: the pages that
+    hold them are not given back when the window has passed them."""
 
     kv_heads: int
     head_dim: int
@@ -19,6 +21,7 @@ class PagedKVSpec:
     page_tokens: int | None = None
     value_dim: int | None = None
     dtype: str | None = None
+    keep_first: int = 0
 
 
 @dataclass(frozen=True)

@@ -7,10 +7,10 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
                       const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
                       int nq, int nkv, int hd, int page_size, int num_pages, ScoreStage st, float scale, int max_tile_ctx,
-                      float* workspace, bool single);
+                      float* workspace, bool single, bool plain);
 size_t attention_generic_workspace_floats(int dtype, int page_size, int n_tiles, int nq, int nkv, int hd, int max_tile_ctx,
-                                          bool single);
-int attention_generic_tile_q(int dtype, int nq, int nkv, int hd, int page_size);
+                                          bool single, bool plain);
+int attention_generic_tile_q(int dtype, int nq, int nkv, int hd, int page_size, bool plain);
 bool attention_mfma_supports(int hd, int page_size, int nq, int nkv);
 bool attention_mfma_decode_supports(int nq, int nkv);
 int attention_mfma_tile_q(int hd);
@@ -31,7 +31,8 @@ int attention_mfma_decode_project(hipStream_t s, const void* q, int q_stride, co
 
 using namespace sprout;
 
-// kernel_kind: 0 = the engine's choice, 1 = the float32-arithmetic kernel.
+// kernel_kind: 0 = the engine's choice, 1 = the float32-arithmetic path (on the matrix cores' float32 instruction where
+// they take the sizes), 2 = the float32-arithmetic kernel on the vector units and no other.
 static bool use_mfma(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind) {
   return kernel_kind == 0 && dtype == kBF16 && nkv > 0 && nq % nkv == 0 && attention_mfma_supports(hd, page_size, nq, nkv);
 }
@@ -45,7 +46,7 @@ extern "C" int sp_attention_plan(int dtype, int hd, int page_size, int nq, int n
     plan[0] = attention_mfma_tile_q(hd);
     plan[1] = attention_mfma_decode_supports(nq, nkv) ? 0 : 1;
   } else {
-    plan[0] = attention_generic_tile_q(dtype, nq, nkv, hd, page_size);
+    plan[0] = attention_generic_tile_q(dtype, nq, nkv, hd, page_size, kernel_kind == 2);
     plan[1] = 1;
   }
   return 0;
@@ -61,7 +62,8 @@ static int64_t workspace_floats_of(int hd, int page_size, int nq, int nkv, int n
 extern "C" int64_t sp_attention_workspace_floats(int dtype, int hd, int page_size, int nq, int nkv, int kernel_kind,
                                                  int n_decode, int max_decode_ctx, int n_tiles, int max_tile_ctx) {
   if (!use_mfma(dtype, hd, page_size, nq, nkv, kernel_kind))   // (n_decode == n_tiles: every sequence brings one query)
-    return (int64_t)attention_generic_workspace_floats(dtype, page_size, n_tiles, nq, nkv, hd, max_tile_ctx, n_decode > 0 && n_decode == n_tiles);
+    return (int64_t)attention_generic_workspace_floats(dtype, page_size, n_tiles, nq, nkv, hd, max_tile_ctx, n_decode > 0 && n_decode == n_tiles,
+                                                       kernel_kind == 2);
   return workspace_floats_of(hd, page_size, nq, nkv, n_decode, max_decode_ctx, n_tiles, max_tile_ctx);
 }
 
@@ -72,10 +74,12 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
                             const int32_t* decode_seqs, int n_decode, int max_decode_ctx, float* workspace,
                             int64_t workspace_floats, void* out, int nq,
                             int nkv, int hd, int page_size, int num_pages, int window, float scale, int kernel_kind,
-                            int scores, float softcap, const float* sinks, int mask_chunk) {
+                            int scores, float softcap, const float* sinks, int mask_chunk, int keep_first) {
   SP_REQUIRE(scores == 0 || (scores == 1 && softcap > 0.f), "sp_attention: no kernel for score stage %d (0 = the scaled product alone, 1 = capped by a positive number)", scores);
   SP_REQUIRE(mask_chunk >= 0, "sp_attention: blocks of %d positions", mask_chunk);
-  const ScoreStage st = {window, mask_chunk, scores == 1 ? softcap : 0.f, sinks};
+  SP_REQUIRE(keep_first >= 0 && (keep_first == 0 || kernel_kind == 2),
+             "sp_attention: %d kept first keys need kernel kind 2, the one kernel that knows them", keep_first);
+  const ScoreStage st = {window, mask_chunk, scores == 1 ? softcap : 0.f, sinks, keep_first};
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_attention: unsupported dtype %d", dtype);
   SP_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "sp_attention: %d query heads do not divide into %d groups", nq, nkv);
   SP_REQUIRE(hd > 0 && hd <= 512, "sp_attention: head size %d is outside 1..512", hd);
@@ -93,13 +97,14 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
     if (n_tiles == 0) return 0;
     SP_REQUIRE(max_tile_ctx >= 0, "sp_attention: negative context length");
     const bool single = n_decode > 0 && n_decode == n_tiles;
-    const int64_t need = (int64_t)attention_generic_workspace_floats(dtype, page_size, n_tiles, nq, nkv, hd, max_tile_ctx, single);
+    const int64_t need = (int64_t)attention_generic_workspace_floats(dtype, page_size, n_tiles, nq, nkv, hd, max_tile_ctx, single,
+                                                                     kernel_kind == 2);
     SP_REQUIRE(need == 0 || (workspace && workspace_floats >= need),
                "sp_attention: workspace of %lld floats is smaller than the %lld needed", (long long)workspace_floats,
                (long long)need);
     return attention_generic(s, dtype, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len,
                              ctx_len, tiles, n_tiles, out, nq, nkv, hd, page_size, num_pages, st, scale,
-                             max_tile_ctx, need ? workspace : nullptr, single);
+                             max_tile_ctx, need ? workspace : nullptr, single, kernel_kind == 2);
   }
   if (plan[1]) {      // groups too large for the one-query kernel: the tile list holds every sequence, and that a step
     n_decode = 0;     // brings one query a sequence (n_decode == n_tiles) is a hint this kernel has no use for

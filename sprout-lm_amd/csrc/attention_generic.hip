@@ -35,7 +35,7 @@ struct Divider {
 
 struct TileSource {
   const int32_t* bt;
-  int nkv, g, hd, page_size, num_pages, max_blocks, k_lo, k_end;
+  int nkv, g, hd, page_size, num_pages, max_blocks, k_lo, k_end, keep;
   Divider by_hd, by_page;
 };
 
@@ -49,7 +49,7 @@ __device__ __forceinline__ void load_tile(const TileSource& src, const T* __rest
       int jj = i % AK, d = i / AK;
       if (!VALUES) src.by_hd.divmod(i, jj, d);
       const int j = kb + jj;
-      if (j >= src.k_lo && j < src.k_end) {
+      if ((j >= src.k_lo || j < src.keep) && j < src.k_end) {
         int logical, slot;
         src.by_page.divmod(j, logical, slot);
         const int page = logical < src.max_blocks ? src.bt[logical] : -1;   // never past the sequence's table row
@@ -116,6 +116,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   // one past the last visible key of the tile (GROUPED: its rows are heads of one query, at pos0)
   src.k_end = pos0 + (GROUPED ? 1 : nvalid);
   src.k_lo = first_visible(pos0, st.window, st.chunk);        // the oldest key any row of the tile sees
+  src.keep = st.keep;                                         // beside the sequence's first `keep` keys, which every row sees
   const int my_lo = first_visible(my_pos, st.window, st.chunk);
   const int n_chunks = gridDim.z, first_key = blockIdx.z * chunk;   // this block's keys: first_key .. + chunk - 1
   if (blockIdx.z + 1 < n_chunks) src.k_end = min(src.k_end, first_key + chunk);   // the last chunk: all that is left
@@ -132,12 +133,17 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   // The keys and values of a tile are requested while the tile before it is still being summed: the walk
   // waits for memory once per tile, not once per element.
   float ktile[2 * MAXD], vtile[2 * MAXD];
-  const int kb0 = max((k_lo / AK) * AK, first_key);
+  // the walk: the tiles that hold kept first keys, then from the window's first tile on; the tiles between are skipped
+  // (their pages may have been given back)
+  const int lo_tile = (k_lo / AK) * AK;
+  const int keep_end = st.keep > 0 ? min(((st.keep + AK - 1) / AK) * AK, lo_tile) : lo_tile;
+  auto skip = [&](int kb) { return kb >= keep_end && kb < lo_tile ? lo_tile : kb; };
+  const int kb0 = skip(max(st.keep > 0 ? 0 : lo_tile, first_key));
   if (kb0 < k_end) {
     load_tile<T, MAXD, false>(src, k_pool, kb0, ktile);
     load_tile<T, MAXD, true>(src, v_pool, kb0, vtile);
   }
-  for (int kb = kb0; kb < k_end; kb += AK) {
+  for (int kb = kb0; kb < k_end; kb = skip(kb + AK)) {
     __syncthreads();  // Qs written / previous V tile consumed
     store_tile<MAXD, false>(KVs, hd, src.by_hd, ktile);
     __syncthreads();
@@ -149,7 +155,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       float dot = 0.f;
 #pragma unroll 8   // several LDS reads on their way at a time; the order of the sum stays
       for (int d = 0; d < hd; ++d) dot = fmaf(Qs[r * kv_stride + d], KVs[c * kv_stride + d], dot);
-      const bool visible = r < nvalid && j >= my_lo && j <= my_pos;
+      const bool visible = r < nvalid && (j >= my_lo || j < st.keep) && j <= my_pos;
       dot *= scale;
       if (st.cap > 0.f) dot = st.cap * tanhf(dot / st.cap);
       s[u] = visible ? dot : -INFINITY;
@@ -176,9 +182,9 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
     Ps[r * PS + c16 + 16] = p[1];
     __syncthreads();  // scores done with the K tile; Ps complete
     store_tile<MAXD, true>(KVs, hd, src.by_hd, vtile);
-    if (kb + AK < k_end) {
-      load_tile<T, MAXD, false>(src, k_pool, kb + AK, ktile);
-      load_tile<T, MAXD, true>(src, v_pool, kb + AK, vtile);
+    if (skip(kb + AK) < k_end) {
+      load_tile<T, MAXD, false>(src, k_pool, skip(kb + AK), ktile);
+      load_tile<T, MAXD, true>(src, v_pool, skip(kb + AK), vtile);
     }
     __syncthreads();
 #pragma unroll
@@ -260,15 +266,16 @@ int attention_f32_tiles(hipStream_t s, const void* q, int q_stride, const void* 
 // Float32 storage goes to the matrix-core kernels of attention_f32.hip where they take the sizes: a step of
 // one-query sequences to the one that shares a sequence's keys out over blocks, any other to the one that walks
 // tiles of 32 queries.
-bool attention_generic_on_matrix_cores(int dtype, int nq, int nkv, int hd, int page_size) {
-  return dtype == kF32 && attention_f32_decode_takes(hd, page_size, nq, nkv);
+// `plain`: the caller asks for the float32-arithmetic kernel of this file and no other (a mask that only it knows).
+bool attention_generic_on_matrix_cores(int dtype, int nq, int nkv, int hd, int page_size, bool plain) {
+  return !plain && dtype == kF32 && attention_f32_decode_takes(hd, page_size, nq, nkv);
 }
-static bool f32_one_query(int dtype, bool single, int nq, int nkv, int hd, int page_size) {
-  return single && attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size);
+static bool f32_one_query(int dtype, bool single, int nq, int nkv, int hd, int page_size, bool plain) {
+  return single && attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size, plain);
 }
 // Queries in a tile of the tile list that the kernels of this path expect.
-int attention_generic_tile_q(int dtype, int nq, int nkv, int hd, int page_size) {
-  return attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size) ? 32 : AQ;
+int attention_generic_tile_q(int dtype, int nq, int nkv, int hd, int page_size, bool plain) {
+  return attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size, plain) ? 32 : AQ;
 }
 
 // How the keys of a step are shared out: {chunks, keys per chunk}.  One chunk unless the step has few blocks
@@ -286,9 +293,9 @@ static void generic_chunks(int n_tiles, int rows_of_blocks, int max_tile_ctx, in
 static bool generic_grouped(bool single, int nq, int nkv) { return single && nkv > 0 && nq % nkv == 0 && nq / nkv > 1 && nq / nkv <= AQ; }
 
 size_t attention_generic_workspace_floats(int dtype, int page_size, int n_tiles, int nq, int nkv, int hd, int max_tile_ctx,
-                                          bool single) {
-  if (f32_one_query(dtype, single, nq, nkv, hd, page_size)) return attention_f32_decode_workspace_floats(n_tiles, nq, hd, max_tile_ctx);
-  if (attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size)) return 0;
+                                          bool single, bool plain) {
+  if (f32_one_query(dtype, single, nq, nkv, hd, page_size, plain)) return attention_f32_decode_workspace_floats(n_tiles, nq, hd, max_tile_ctx);
+  if (attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size, plain)) return 0;
   int n_chunks, chunk;
   generic_chunks(n_tiles, generic_grouped(single, nq, nkv) ? nkv : nq, max_tile_ctx, &n_chunks, &chunk);
   return n_chunks > 1 ? size_t(n_tiles) * AQ * nq * n_chunks * (hd + 2) : 0;
@@ -347,14 +354,15 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
                       const void* v_pool, const int32_t* block_tables, int max_blocks, const int32_t* q_start,
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
                       int nq, int nkv, int hd, int page_size, int num_pages, ScoreStage st, float scale, int max_tile_ctx,
-                      float* workspace, bool single) {
+                      float* workspace, bool single, bool plain) {
+  SP_REQUIRE(plain || st.keep == 0, "sp_attention: kept first keys are known to the float32-arithmetic kernel alone");
   SP_REQUIRE(int64_t(max_blocks) * page_size < (int64_t(1) << 24),
              "sp_attention: block tables of %d pages of %d tokens exceed the 2^24 positions this kernel counts",
              max_blocks, page_size);
-  if (f32_one_query(dtype, single, nq, nkv, hd, page_size))
+  if (f32_one_query(dtype, single, nq, nkv, hd, page_size, plain))
     return attention_f32_decode(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, ctx_len, tiles, n_tiles,
                                 out, nq, nkv, hd, page_size, num_pages, st, scale, max_tile_ctx, workspace);
-  if (attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size))
+  if (attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size, plain))
     return attention_f32_tiles(s, q, q_stride, k_pool, v_pool, block_tables, max_blocks, q_start, q_len, ctx_len, tiles,
                                n_tiles, out, nq, nkv, hd, page_size, num_pages, st, scale);
   if (dtype == kF32)

@@ -65,6 +65,7 @@ struct ScoreStage {
   int chunk;           // > 0: only keys of the query's own block of `chunk` positions, counted from position 0
   float cap;           // > 0: the scaled score s becomes cap * tanh(s / cap)
   const float* sinks;  // one number per query head whose exponential joins the softmax's denominator (null: none)
+  int keep;            // > 0: the sequence's first `keep` keys stay visible to every later query, whatever the window
 };
 // The first key that a query at `pos` sees.
 __device__ __forceinline__ int first_visible(int pos, int window, int chunk) {

@@ -9,7 +9,7 @@ namespace sprout {
 // The `top` largest of a token's `experts` logits (the lowest index wins a tie), in falling order, and the softmax
 // over the chosen logits alone.
 __device__ __forceinline__ void route_token(const float* __restrict__ z, int experts, int top, int32_t* __restrict__ id,
-                                            float* __restrict__ w) {
+                                            float* __restrict__ w, bool sigmoid = false) {
   // the k-th choice is the largest logit that comes after the (k-1)-th in the order (falling value, rising index):
   // nothing already written is read back
   float prev_z = INFINITY, top_z = 0.f, sum = 0.f;
@@ -24,14 +24,14 @@ __device__ __forceinline__ void route_token(const float* __restrict__ z, int exp
     }
     if (best < 0) best = (prev + 1) % experts;      // only where logits are not numbers
     if (k == 0) top_z = best_z;
-    const float ex = expf(best_z - top_z);
+    const float ex = sigmoid ? 1.0f / (1.0f + expf(-best_z)) : expf(best_z - top_z);
     sum += ex;
     id[k] = best;
     w[k] = ex;
     prev = best;
     prev_z = best_z;
   }
-  const float scale = 1.0f / sum;
+  const float scale = sigmoid ? 1.0f : 1.0f / sum;
   for (int k = 0; k < top; ++k) w[k] *= scale;
 }
 
@@ -39,7 +39,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ z, int exp
 // coalesced load, and every choice is a reduction over the wave (larger value first, lower index among equals).
 constexpr int kWaveExperts = 256;
 __device__ __forceinline__ void route_token_wave(const float* __restrict__ z, int experts, int top, int32_t* __restrict__ id,
-                                                 float* __restrict__ w, int lane) {
+                                                 float* __restrict__ w, int lane, bool sigmoid = false) {
   constexpr int J = kWaveExperts / 64, NONE = 0x7fffffff;
   float v[J];
   unsigned taken = 0;
@@ -65,13 +65,13 @@ __device__ __forceinline__ void route_token_wave(const float* __restrict__ z, in
     }
     if ((be & 63) == lane) taken |= 1u << (be >> 6);
     if (k == 0) top_z = bv;
-    const float ex = expf(bv - top_z);
+    const float ex = sigmoid ? 1.0f / (1.0f + expf(-bv)) : expf(bv - top_z);
     sum += ex;
 #pragma unroll
     for (int j = 0; j < J; ++j)
       if (k == lane + 64 * j) { my_id[j] = be; my_ex[j] = ex; }
   }
-  const float scale = 1.0f / sum;
+  const float scale = sigmoid ? 1.0f : 1.0f / sum;
 #pragma unroll
   for (int j = 0; j < J; ++j)
     if (lane + 64 * j < top) { id[lane + 64 * j] = my_id[j]; w[lane + 64 * j] = my_ex[j] * scale; }
@@ -82,6 +82,7 @@ __device__ __forceinline__ void route_token_wave(const float* __restrict__ z, in
 //   mode 1: scores = the softmax over all outputs; the choice goes by score + correction[e], and only among the outputs
 //           of the `keep` groups (of `groups` equal groups of neighbours) whose best such sum is largest; weights = the
 //           chosen outputs' scores (without the correction) times `scale`, not renormalised.  Up to 256 outputs.
+//   mode 2: the `top` largest logits; weights = the sigmoid of each chosen logit, not renormalised.
 struct RouteRule {
   int mode;
   const float* correction;
@@ -173,12 +174,13 @@ __global__ void route_topk_kernel(const float* __restrict__ logits, long long st
     const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (t >= T) return;
     if (rule.mode == 1) route_token_scored(logits + size_t(t) * stride, experts, top, rule, ids + size_t(t) * top, weights + size_t(t) * top, threadIdx.x & 63);
-    else route_token_wave(logits + size_t(t) * stride, experts, top, ids + size_t(t) * top, weights + size_t(t) * top, threadIdx.x & 63);
+    else route_token_wave(logits + size_t(t) * stride, experts, top, ids + size_t(t) * top, weights + size_t(t) * top, threadIdx.x & 63,
+                          rule.mode == 2);
     return;
   }
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
-  route_token(logits + size_t(t) * stride, experts, top, ids + size_t(t) * top, weights + size_t(t) * top);
+  route_token(logits + size_t(t) * stride, experts, top, ids + size_t(t) * top, weights + size_t(t) * top, rule.mode == 2);
 }
 
 // One block: sorts the pairs (token, choice) by expert.  row_of_pair[p] = the row of pair p in the sorted order,
@@ -206,10 +208,11 @@ __global__ __launch_bounds__(1024) void route_sort_kernel(const float* __restric
         route_token_scored(logits + size_t(t) * stride, experts, top, rule, ids + size_t(t) * top, weights + size_t(t) * top, lane);
     else if (experts <= kWaveExperts)
       for (int t = wave; t < pairs / top; t += waves)
-        route_token_wave(logits + size_t(t) * stride, experts, top, ids + size_t(t) * top, weights + size_t(t) * top, lane);
+        route_token_wave(logits + size_t(t) * stride, experts, top, ids + size_t(t) * top, weights + size_t(t) * top, lane,
+                         rule.mode == 2);
     else
       for (int t = threadIdx.x; t < pairs / top; t += blockDim.x)
-        route_token(logits + size_t(t) * stride, experts, top, ids + size_t(t) * top, weights + size_t(t) * top);
+        route_token(logits + size_t(t) * stride, experts, top, ids + size_t(t) * top, weights + size_t(t) * top, rule.mode == 2);
   }
   __syncthreads();
   const int chunks = (pairs + 63) / 64, per_wave = (chunks + waves - 1) / waves;
@@ -275,7 +278,7 @@ __global__ __launch_bounds__(256) void route_combine_kernel(const float* __restr
     if (i >= H) return;
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int k = 0; k < top; ++k) {
-      const float w = wt[k];
+      const float w = weights ? wt[k] : 1.0f;
       float4 v;
       if (id && id[k] >= real) v = make_float4(to_float(own[i]), to_float(own[i + 1]), to_float(own[i + 2]), to_float(own[i + 3]));
       else v = *reinterpret_cast<const float4*>(y + size_t(rows[k]) * H + i);
@@ -288,7 +291,7 @@ __global__ __launch_bounds__(256) void route_combine_kernel(const float* __restr
   }
   for (int i = blockIdx.y * 1024 + threadIdx.x; i < min(H, (int(blockIdx.y) + 1) * 1024); i += 256) {
     float sum = 0.f;
-    for (int k = 0; k < top; ++k) sum = fmaf(wt[k], id && id[k] >= real ? to_float(own[i]) : y[size_t(rows[k]) * H + i], sum);
+    for (int k = 0; k < top; ++k) sum = fmaf(weights ? wt[k] : 1.0f, id && id[k] >= real ? to_float(own[i]) : y[size_t(rows[k]) * H + i], sum);
     residual[size_t(t) * H + i] += sum;
   }
 }
@@ -347,6 +350,14 @@ extern "C" int sp_route(void* stream, const float* logits, int32_t* ids, float* 
                       pair_of_row, tiles, n_tiles, RouteRule{0, nullptr, 1, 1, 1.f}, "sp_route");
 }
 
+extern "C" int sp_route_sigmoid(void* stream, const float* logits, int32_t* ids, float* weights, int T, int experts, int top,
+                                int tile_rows, int32_t* row_of_pair, int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles) {
+  SP_REQUIRE(T >= 0 && experts > 0 && experts <= 960 && top > 0 && top <= experts && tile_rows > 0, "sp_route_sigmoid: bad sizes");
+  SP_REQUIRE(logits && ids && weights && row_of_pair && pair_of_row && tiles && n_tiles, "sp_route_sigmoid: null operand");
+  return route_launch((hipStream_t)stream, logits, experts, ids, weights, T, experts, experts, top, tile_rows, row_of_pair,
+                      pair_of_row, tiles, n_tiles, RouteRule{2, nullptr, 1, 1, 1.f}, "sp_route_sigmoid");
+}
+
 extern "C" int sp_route_scored(void* stream, const float* logits, long long stride, const float* correction, int groups,
                                int keep, float scale, int32_t* ids, float* weights, int T, int outputs, int real, int top,
                                int tile_rows, int32_t* row_of_pair, int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles) {
@@ -362,7 +373,7 @@ extern "C" int sp_route_scored(void* stream, const float* logits, long long stri
 
 extern "C" int sp_route_combine(void* stream, const float* y, const int32_t* row_of_pair, const float* weights, int top,
                                 float* residual, int T, int H) {
-  SP_REQUIRE(T >= 0 && H > 0 && top > 0 && y && row_of_pair && weights && residual, "sp_route_combine: bad arguments");
+  SP_REQUIRE(T >= 0 && H > 0 && top > 0 && y && row_of_pair && residual, "sp_route_combine: bad arguments");
   if (T == 0) return 0;
   route_combine_kernel<float><<<dim3(T, (H + 1023) / 1024), 256, 0, (hipStream_t)stream>>>(y, row_of_pair, weights, top, residual, H,
                                                                                            nullptr, nullptr, 0);

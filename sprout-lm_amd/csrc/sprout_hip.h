@@ -104,7 +104,8 @@ int sp_attention(void* stream, int dtype, const void* q, int q_stride, const voi
                  int max_tile_ctx, int mean_tile_walk, const int32_t* decode_seqs, int n_decode, int max_decode_ctx,
                  float* workspace, int64_t workspace_floats, void* out, int nq, int nkv, int hd, int page_size,
                  int num_pages, int window, float scale, int kernel_kind, int scores, float softcap, const float* sinks,
-                 int mask_chunk);
+                 int mask_chunk, int keep_first);
+// keep_first > 0: a sequence's first keep_first keys stay visible to every later query beside its window (kernel_kind 2 only).
 
 // A step of one-query sequences only (bfloat16): attention with the output projection folded into the merge
 // of the key chunks: residual[q_start[seq], :] += attention(seq) . w_o^T with w_o [hidden, nq * hd] bfloat16
@@ -245,6 +246,10 @@ int sp_route(void* stream, const float* logits, int32_t* ids, float* weights, in
              int32_t* row_of_pair, int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles);
 int sp_route_combine(void* stream, const float* y, const int32_t* row_of_pair, const float* weights, int top,
                      float* residual, int T, int H);
+// sp_route whose weights are the sigmoid of each chosen logit, not renormalised.  (sp_route_combine with null weights adds
+// the rows as they are.)
+int sp_route_sigmoid(void* stream, const float* logits, int32_t* ids, float* weights, int T, int experts, int top, int tile_rows,
+                     int32_t* row_of_pair, int32_t* pair_of_row, int32_t* tiles, int32_t* n_tiles);
 // sp_route with another rule of choice: scores = the softmax over all `outputs` logits of a token (rows `stride`
 // apart); the choice goes by score + correction[e] (null: none) and only among the outputs of the `keep` of `groups`
 // equal groups of neighbours whose best such sum is largest (the lower index wins every tie); weights = the chosen
@@ -291,4 +296,56 @@ int sp_retention(void* stream, int dtype, const void* proj, long long stride, in
                  float* scratch);
 // max_q_len, scratch: as for sp_rglru, with sp_retention_scratch_floats numbers.
 long long sp_retention_scratch_floats(int heads, int dim, int vdim, int n_seqs, int max_q_len, int T);
+
+// ---- short causal convolutions, state-space scans and what goes with them (ssm.hip) ----
+// y[t, c] = act(bias[c] + sum_j w[c, j] x[t - taps + 1 + j, c]) (+ x[t, c] with add_input), a causal convolution over
+// time per channel within each request; inputs before a request's share of the step come from its state rows
+// [slots, taps - 1, channels] (float32, oldest first; zeros in a fresh slot), which are left holding the request's last
+// taps - 1 inputs.  x [T, x_stride] from column x_off on, out [T, out_stride] from out_off on, both of `dtype`, not the
+// same memory; w [channels, taps] and bias (may be null) of w_dtype.  act 0: none, 1: SiLU.  taps 1: no state.
+int sp_short_conv(void* stream, int dtype, const void* x, long long x_stride, int x_off, int channels, int taps, int w_dtype,
+                  const void* w, const void* bias, int act, int add_input, void* out, long long out_stride, int out_off,
+                  const int32_t* q_start, const int32_t* q_len, const int32_t* seq_of_token, const int32_t* state_slots,
+                  float* state, int T, int n_seqs);
+// out [T, parts * size] = x / sqrt(mean over each part of x^2 + eps) * w, every row in `parts` equal parts, x float32.
+int sp_group_rmsnorm(void* stream, const float* x, int w_dtype, const void* w, float eps, int out_dtype, void* out, int T,
+                     int parts, int size);
+// In place on n numbers of `dtype`: kind 0 = x * Phi(x), the exact (erf) GELU.
+int sp_activation(void* stream, int dtype, void* x, long long n, int kind);
+// out[p, :] = x[p / top, :] * weights[p]   (p < T * top; x, out of `dtype` [.., H]; weights float32)
+int sp_scale_rows(void* stream, int dtype, const void* x, const float* weights, int top, void* out, int T, int H);
+// State-space duality scan (Mamba-2).  Per head n (group n / (heads / groups)) and token t of a request:
+//   d = softplus(dt[t, n] + dt_bias[n]),  S <- exp(-exp(a_log[n]) d) S + d B_t u_t^T,  y_t = S^T C_t + skip[n] u_t,
+// and out[t] = y_t * silu(z_t), float32 [T, heads * vdim].  z and dt are columns of proj [T, proj_stride] (z_off, dt_off);
+// u (heads * vdim), B and C (groups * state each) are the columns of xbc [T, xbc_stride] in that order, of `dtype`.
+// state float32 [slots, heads, state, vdim].  dt_bias, a_log, skip float32 [heads].  state up to 256.
+int sp_ssd_scan(void* stream, int dtype, const void* proj, long long proj_stride, int z_off, int dt_off, const void* xbc,
+                long long xbc_stride, int heads, int vdim, int state_size, int groups, const float* dt_bias, const float* a_log,
+                const float* skip, const int32_t* q_start, const int32_t* q_len, const int32_t* state_slots, float* state,
+                float* out, int T, int n_seqs);
+// Selective scan (Mamba).  Per channel c and token t: d = softplus(dt[t, c]) (dt float32 [T, inner], bias included),
+//   S[c, :] <- exp(d a[c, :]) S[c, :] + d u[t, c] B_t,  y = S[c, :] . C_t + skip[c] u[t, c],  out[t, c] = y * silu(z[t, c]).
+// u [T, u_stride] from u_off, z likewise, B and C (state numbers each) the columns of bc [T, bc_stride] from bc_off on, all
+// of `dtype`; a float32 [inner, state] (negative), skip float32 [inner]; state float32 [slots, inner, state]; out of
+// `dtype` [T, inner].  state up to 256.
+int sp_selective_scan(void* stream, int dtype, const void* u, long long u_stride, int u_off, const void* z, long long z_stride,
+                      int z_off, const float* dt, const void* bc, long long bc_stride, int bc_off, int inner, int state_size,
+                      const float* a, const float* skip, const int32_t* q_start, const int32_t* q_len,
+                      const int32_t* state_slots, float* state, void* out, int T, int n_seqs);
+// Queries and keys of attention whose heads' weights are mixed after the softmax.  qk [T, (nq + nkv) * dim] of `dtype`
+// holds q then k.  Every head is divided by its root mean square (eps inside the root) and multiplied by q_norm or k_norm
+// (dim numbers of w_dtype), then the first rotary_dim numbers turn, 2i with 2i + 1, by positions[t] * freq[i] (float64
+// table; the angle is float64 for float32 storage, float32 otherwise).  The values are the keys as they came in.  For the
+// attention kernels, which tie a value head to a key head, every (query head g, value head c) pair becomes a head of its
+// own: query row [(kv(g) * nkv + c) * (nq / nkv) + g % (nq / nkv)] = q_g, key head [a * nkv + c] = k_a, value head
+// [a * nkv + c] = v_c, at `width` numbers a head, zeros behind dim.  Keys and values go into the pools (nkv * nkv heads) at
+// slot_mapping[t] (negative: not written), queries to q_out [T, nq * nkv * width].
+int sp_qk_cross_prepare(void* stream, int dtype, const void* qk, int nq, int nkv, int dim, int width, int w_dtype,
+                        const void* q_norm, const void* k_norm, float eps, const int32_t* positions, const double* freq,
+                        int rotary_dim, const int32_t* slot_mapping, void* q_out, void* k_pool, void* v_pool, int page_size,
+                        int T);
+// out[t, h, :dim] = sum_g talk[h, g] * o[t, (kv(g) * nkv + kv(h)) * (nq / nkv) + g % (nq / nkv), :dim], o [T, nq * nkv * width]:
+// the outputs of the heads made by sp_qk_cross_prepare, mixed by talk (float32 [nq, nq]).  out [T, nq * dim], both `dtype`.
+int sp_head_mix(void* stream, int dtype, const void* o, const float* talk, int nq, int nkv, int dim, int width, void* out,
+                int T);
 }

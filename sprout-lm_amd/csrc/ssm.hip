@@ -1,0 +1,497 @@
+// Short causal convolutions with per-request state, the scans of two state-space mixers (the state-space-duality form
+// with one decay per head and token, and the selective scan with one decay per channel, state and token), and what
+// attention with weights mixed between heads after the softmax needs around the attention kernels.  Step sizes, decays,
+// their exponentials, the states and all norms are float32 whatever the storage type; only loads of projections and
+// weights and the stores of results see it.  A step's tokens lie flat, request after request; q_start / q_len /
+// state_slots (one entry per request of the step) say where a request's tokens are and which row of the state tensors is
+// its own.  A kernel reads the state as the step before left it and leaves it for the next one, so a portion of a prompt
+// and a single decoded token are the same call.
+#include "common.h"
+#include "sprout_hip.h"
+
+namespace sprout {
+
+__device__ __forceinline__ float softplus_of(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+__device__ __forceinline__ float silu_of(float z) { return z / (1.0f + expf(-z)); }
+
+// ------------------------------------------------------------------------------------------------ short convolution
+struct ConvArgs {
+  const void* x;
+  long long x_stride;
+  int x_off, channels, taps;
+  const void* w;
+  const void* bias;
+  int act, add_input;
+  void* out;
+  long long out_stride;
+  int out_off;
+  const int32_t* q_start;
+  const int32_t* q_len;
+  const int32_t* seq_of_token;
+  const int32_t* state_slots;
+  float* state;
+};
+
+// A thread a (token, channel): the taps in their order, inputs before the request's share of the step from its state rows.
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void short_conv_kernel(ConvArgs a) {
+  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= a.channels) return;
+  const int s = a.seq_of_token[t];
+  const int j = t - a.q_start[s], keep = a.taps - 1;
+  const T* x = (const T*)a.x + a.x_off + c;
+  const TW* w = (const TW*)a.w + size_t(c) * a.taps;
+  const float* rows = keep ? a.state + size_t(a.state_slots[s]) * keep * a.channels + c : nullptr;
+  float acc = a.bias ? to_float(((const TW*)a.bias)[c]) : 0.f;
+  for (int tap = 0; tap < a.taps; ++tap) {
+    const int back = keep - tap;
+    const float v = j - back >= 0 ? to_float(x[size_t(t - back) * a.x_stride]) : rows[size_t(keep + j - back) * a.channels];
+    acc = fmaf(to_float(w[tap]), v, acc);
+  }
+  if (a.act == 1) acc = silu_of(acc);
+  if (a.add_input) acc += to_float(x[size_t(t) * a.x_stride]);
+  ((T*)a.out)[size_t(t) * a.out_stride + a.out_off + c] = from_float<T>(acc);
+}
+
+// A thread a (request, channel): the state rows become the last taps - 1 inputs, older ones moved up from the rows
+// themselves where the request brought fewer tokens than that.  Rows are written oldest first and read at or behind
+// the row being written, by the one thread that owns the channel.
+template <typename T>
+__global__ __launch_bounds__(256) void short_conv_state_kernel(ConvArgs a) {
+  const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= a.channels) return;
+  const int L = a.q_len[s], keep = a.taps - 1;
+  if (L <= 0) return;
+  const T* x = (const T*)a.x + size_t(a.q_start[s]) * a.x_stride + a.x_off + c;
+  float* rows = a.state + size_t(a.state_slots[s]) * keep * a.channels + c;
+  for (int j = 0; j < keep; ++j) {
+    const int src = L - keep + j;
+    rows[size_t(j) * a.channels] = src >= 0 ? to_float(x[size_t(src) * a.x_stride]) : rows[size_t(j + L) * a.channels];
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ small kernels
+template <typename TW, typename TO>
+__global__ __launch_bounds__(256) void group_rmsnorm_kernel(const float* __restrict__ x, const TW* __restrict__ w, float eps,
+                                                            TO* __restrict__ out, int parts, int size) {
+  __shared__ float scratch[16];
+  const size_t row = blockIdx.x;
+  const int part = int(row % parts);
+  const float* xr = x + row * size;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < size; i += 256) ss = fmaf(xr[i], xr[i], ss);
+  const float r = 1.0f / sqrtf(block_sum(ss, scratch) / float(size) + eps);
+  for (int i = threadIdx.x; i < size; i += 256)
+    out[row * size + i] = from_float<TO>(xr[i] * r * to_float(w[size_t(part) * size + i]));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_erf_kernel(T* __restrict__ x, long long n) {
+  for (long long i = blockIdx.x * 256ll + threadIdx.x; i < n; i += 256ll * gridDim.x) {
+    const float v = to_float(x[i]);
+    x[i] = from_float<T>(0.5f * v * (1.0f + erff(v * 0.70710678118654752f)));
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void scale_rows_kernel(const T* __restrict__ x, const float* __restrict__ weights, int top,
+                                                         T* __restrict__ out, int H) {
+  const size_t p = blockIdx.x;
+  const float w = weights[p];
+  const T* src = x + (p / top) * H;
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < H; i += 256 * gridDim.y) out[p * H + i] = from_float<T>(to_float(src[i]) * w);
+}
+
+// ------------------------------------------------------------------------------------------------ state-space duality scan
+struct SsdArgs {
+  const void* proj;
+  long long proj_stride;
+  int z_off, dt_off;
+  const void* xbc;
+  long long xbc_stride;
+  int heads, vdim, state_size, groups;
+  const float* dt_bias;
+  const float* a_log;
+  const float* skip;
+  const int32_t* q_start;
+  const int32_t* q_len;
+  const int32_t* state_slots;
+  float* state;
+  float* out;
+};
+
+// A block per request and 32 columns of the heads' values; a column's state rows are shared out over 8 neighbouring lanes
+// (lane rg holds rows rg, rg + 8, ...: KPT of them), so a token's output is a sum over those lanes alone and the walk along
+// the request's tokens needs no barrier.  Columns are independent of each other: S[:, p] takes B and u_p only.
+template <typename T, int KPT>
+__global__ __launch_bounds__(256) void ssd_scan_kernel(SsdArgs a) {
+  const int s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rg = lane & 7, pc = lane >> 3;
+  const int inner = a.heads * a.vdim, N = a.state_size;
+  int col = blockIdx.x * 32 + wave * 8 + pc;
+  const bool live = col < inner;
+  if (!live) col = inner - 1;      // the lane stays for its neighbours' sums and stores nothing
+  const int n = col / a.vdim, p = col % a.vdim, g = n / (a.heads / a.groups);
+  const int q0 = a.q_start[s], L = a.q_len[s];
+  if (L <= 0) return;
+  float* S = a.state + ((size_t(a.state_slots[s]) * a.heads + n) * N) * a.vdim + p;
+  float st[KPT];
+#pragma unroll
+  for (int k = 0; k < KPT; ++k) {
+    const int r = rg + 8 * k;
+    st[k] = r < N ? S[size_t(r) * a.vdim] : 0.f;
+  }
+  const float rate = expf(a.a_log[n]), bias = a.dt_bias[n], skip = a.skip[n];
+  const T* proj = (const T*)a.proj;
+  const T* xbc = (const T*)a.xbc;
+  const int b_off = inner + g * N, c_off = inner + a.groups * N + g * N;
+  for (int t = q0; t < q0 + L; ++t) {
+    const T* pr = proj + size_t(t) * a.proj_stride;
+    const T* xr = xbc + size_t(t) * a.xbc_stride;
+    const float d = softplus_of(to_float(pr[a.dt_off + n]) + bias);
+    const float decay = expf(-rate * d);
+    const float u = to_float(xr[col]);
+    const float z = to_float(pr[a.z_off + col]);
+    const float du = d * u;
+    float y = 0.f;
+#pragma unroll
+    for (int k = 0; k < KPT; ++k) {
+      const int r = rg + 8 * k;
+      if (r < N) {
+        st[k] = fmaf(decay, st[k], du * to_float(xr[b_off + r]));
+        y = fmaf(st[k], to_float(xr[c_off + r]), y);
+      }
+    }
+    y += __shfl_xor(y, 1, 64);
+    y += __shfl_xor(y, 2, 64);
+    y += __shfl_xor(y, 4, 64);
+    if (rg == 0 && live) a.out[size_t(t) * inner + col] = fmaf(skip, u, y) * silu_of(z);
+  }
+  if (live) {
+#pragma unroll
+    for (int k = 0; k < KPT; ++k) {
+      const int r = rg + 8 * k;
+      if (r < N) S[size_t(r) * a.vdim] = st[k];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ selective scan
+struct SelArgs {
+  const void* u;
+  long long u_stride;
+  int u_off;
+  const void* z;
+  long long z_stride;
+  int z_off;
+  const float* dt;
+  const void* bc;
+  long long bc_stride;
+  int bc_off, inner, state_size;
+  const float* a;
+  const float* skip;
+  const int32_t* q_start;
+  const int32_t* q_len;
+  const int32_t* state_slots;
+  float* state;
+  void* out;
+};
+
+// A block per request and 64 channels; a channel's states are shared out over 4 neighbouring lanes (lane ng holds states ng,
+// ng + 4, ...: KPT of them).
+template <typename T, int KPT>
+__global__ __launch_bounds__(256) void selective_scan_kernel(SelArgs a) {
+  const int s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ng = lane & 3, cc = lane >> 2;
+  const int N = a.state_size;
+  int c = blockIdx.x * 64 + wave * 16 + cc;
+  const bool live = c < a.inner;
+  if (!live) c = a.inner - 1;
+  const int q0 = a.q_start[s], L = a.q_len[s];
+  if (L <= 0) return;
+  float* S = a.state + (size_t(a.state_slots[s]) * a.inner + c) * N;
+  float st[KPT], ak[KPT];
+#pragma unroll
+  for (int k = 0; k < KPT; ++k) {
+    const int n = ng + 4 * k;
+    st[k] = n < N ? S[n] : 0.f;
+    ak[k] = n < N ? a.a[size_t(c) * N + n] : 0.f;
+  }
+  const float skip = a.skip[c];
+  const T* up = (const T*)a.u + a.u_off + c;
+  const T* zp = (const T*)a.z + a.z_off + c;
+  const T* bc = (const T*)a.bc + a.bc_off;
+  for (int t = q0; t < q0 + L; ++t) {
+    const float d = softplus_of(a.dt[size_t(t) * a.inner + c]);
+    const float u = to_float(up[size_t(t) * a.u_stride]);
+    const float z = to_float(zp[size_t(t) * a.z_stride]);
+    const T* row = bc + size_t(t) * a.bc_stride;
+    const float du = d * u;
+    float y = 0.f;
+#pragma unroll
+    for (int k = 0; k < KPT; ++k) {
+      const int n = ng + 4 * k;
+      if (n < N) {
+        st[k] = fmaf(expf(d * ak[k]), st[k], du * to_float(row[n]));
+        y = fmaf(st[k], to_float(row[N + n]), y);
+      }
+    }
+    y += __shfl_xor(y, 1, 64);
+    y += __shfl_xor(y, 2, 64);
+    if (ng == 0 && live) ((T*)a.out)[size_t(t) * a.inner + c] = from_float<T>(fmaf(skip, u, y) * silu_of(z));
+  }
+  if (live) {
+#pragma unroll
+    for (int k = 0; k < KPT; ++k) {
+      const int n = ng + 4 * k;
+      if (n < N) S[n] = st[k];
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ attention with mixed heads
+struct CrossArgs {
+  const void* qk;
+  int nq, nkv, dim, width;
+  const void* q_norm;
+  const void* k_norm;
+  float eps;
+  const int32_t* positions;
+  const double* freq;
+  int rotary_dim;
+  const int32_t* slot_mapping;
+  void* q_out;
+  void* k_pool;
+  void* v_pool;
+  int page_size;
+};
+
+// A block per (token, head of q or k): the head's norm, the turning of its first numbers in neighbouring pairs, and the
+// copies that make every (query head, value head) pair a head of the attention kernels.
+template <typename T, typename TW, bool F64>
+__global__ __launch_bounds__(128) void qk_cross_prepare_kernel(CrossArgs a) {
+  extern __shared__ float lds[];      // the head as it came [dim], normed [dim], 16 for the sum
+  float* raw = lds;
+  float* normed = lds + a.dim;
+  float* scratch = normed + a.dim;
+  const int t = blockIdx.x, hs = blockIdx.y;
+  const bool is_q = hs < a.nq;
+  const T* src = (const T*)a.qk + (size_t(t) * (a.nq + a.nkv) + hs) * a.dim;
+  float ss = 0.f;
+  for (int d = threadIdx.x; d < a.dim; d += 128) {
+    const float v = to_float(src[d]);
+    raw[d] = v;
+    ss = fmaf(v, v, ss);
+  }
+  const float r = 1.0f / sqrtf(block_sum(ss, scratch) / float(a.dim) + a.eps);
+  const TW* nw = (const TW*)(is_q ? a.q_norm : a.k_norm);
+  for (int d = threadIdx.x; d < a.dim; d += 128) normed[d] = raw[d] * r * to_float(nw[d]);
+  __syncthreads();
+  const int pos = a.positions[t];
+  const int group = a.nq / a.nkv, nkv2 = a.nkv * a.nkv;
+  const int slot = a.slot_mapping ? a.slot_mapping[t] : -1;
+  for (int d = threadIdx.x; d < a.width; d += 128) {
+    float o = 0.f;
+    if (d < a.dim) {
+      o = normed[d];
+      if (d < a.rotary_dim) {
+        float cs, sn;
+        if (F64) {
+          const double angle = double(pos) * a.freq[d >> 1];
+          cs = float(cos(angle));
+          sn = float(sin(angle));
+        } else {
+          sincosf(float(pos) * float(a.freq[d >> 1]), &sn, &cs);
+        }
+        const float other = normed[d ^ 1];
+        o = (d & 1) ? fmaf(o, cs, other * sn) : fmaf(o, cs, -other * sn);
+      }
+    }
+    if (is_q) {
+      const int kv = hs / group, rr = hs % group;
+      T* q_out = (T*)a.q_out + size_t(t) * a.nq * a.nkv * a.width;
+      for (int c = 0; c < a.nkv; ++c) q_out[(size_t(kv * a.nkv + c) * group + rr) * a.width + d] = from_float<T>(o);
+    } else if (slot >= 0) {
+      const int kv = hs - a.nq, page = slot / a.page_size, off = slot % a.page_size;
+      const T value = from_float<T>(d < a.dim ? raw[d] : 0.f);
+      for (int c = 0; c < a.nkv; ++c) {
+        ((T*)a.k_pool)[((size_t(page) * nkv2 + kv * a.nkv + c) * a.page_size + off) * a.width + d] = from_float<T>(o);
+        ((T*)a.v_pool)[((size_t(page) * nkv2 + c * a.nkv + kv) * a.width + d) * a.page_size + off] = value;
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(128) void head_mix_kernel(const T* __restrict__ o, const float* __restrict__ talk, int nq, int nkv,
+                                                       int dim, int width, T* __restrict__ out) {
+  const int t = blockIdx.x, h = blockIdx.y, group = nq / nkv, mine = h / group;
+  const T* row = o + size_t(t) * nq * nkv * width;
+  for (int d = threadIdx.x; d < dim; d += 128) {
+    float sum = 0.f;
+    for (int g = 0; g < nq; ++g)
+      sum = fmaf(talk[h * nq + g], to_float(row[(size_t((g / group) * nkv + mine) * group + g % group) * width + d]), sum);
+    out[(size_t(t) * nq + h) * dim + d] = from_float<T>(sum);
+  }
+}
+
+}  // namespace sprout
+
+using namespace sprout;
+
+extern "C" int sp_short_conv(void* stream, int dtype, const void* x, long long x_stride, int x_off, int channels, int taps,
+                             int w_dtype, const void* w, const void* bias, int act, int add_input, void* out,
+                             long long out_stride, int out_off, const int32_t* q_start, const int32_t* q_len,
+                             const int32_t* seq_of_token, const int32_t* state_slots, float* state, int T, int n_seqs) {
+  SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_short_conv: unsupported dtype %d", dtype);
+  SP_REQUIRE(w_dtype == dtype || w_dtype == kF32, "sp_short_conv: weights of dtype %d beside rows of dtype %d", w_dtype, dtype);
+  SP_REQUIRE(channels > 0 && taps > 0 && taps <= 64 && T >= 0 && n_seqs >= 0, "sp_short_conv: bad sizes (%d channels, %d taps)", channels, taps);
+  SP_REQUIRE(x_off >= 0 && out_off >= 0 && x_stride >= x_off + channels && out_stride >= out_off + channels,
+             "sp_short_conv: %d channels do not fit the rows", channels);
+  SP_REQUIRE(act == 0 || act == 1, "sp_short_conv: no activation %d (0 = none, 1 = SiLU)", act);
+  SP_REQUIRE(x && w && out && x != out && q_start && q_len && seq_of_token && state_slots && (taps == 1 || state),
+             "sp_short_conv: null or aliased operand");
+  if (T == 0 || n_seqs == 0) return 0;
+  const ConvArgs a = {x, x_stride, x_off, channels, taps, w, bias, act, add_input, out, out_stride, out_off,
+                      q_start, q_len, seq_of_token, state_slots, state};
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(T, (channels + 255) / 256);
+  if (dtype == kF32) short_conv_kernel<float, float><<<grid, 256, 0, s>>>(a);
+  else if (w_dtype == kF32) short_conv_kernel<bf16_t, float><<<grid, 256, 0, s>>>(a);
+  else short_conv_kernel<bf16_t, bf16_t><<<grid, 256, 0, s>>>(a);
+  if (check_launch("sp_short_conv")) return 1;
+  if (taps == 1) return 0;
+  const dim3 grid2(n_seqs, (channels + 255) / 256);
+  if (dtype == kF32) short_conv_state_kernel<float><<<grid2, 256, 0, s>>>(a);
+  else short_conv_state_kernel<bf16_t><<<grid2, 256, 0, s>>>(a);
+  return check_launch("sp_short_conv (state)");
+}
+
+extern "C" int sp_group_rmsnorm(void* stream, const float* x, int w_dtype, const void* w, float eps, int out_dtype, void* out,
+                                int T, int parts, int size) {
+  SP_REQUIRE(T >= 0 && parts > 0 && size > 0 && x && w && out, "sp_group_rmsnorm: bad arguments");
+  SP_REQUIRE((w_dtype == kF32 || w_dtype == kBF16) && (out_dtype == kF32 || out_dtype == kBF16), "sp_group_rmsnorm: unsupported dtype");
+  if (T == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned rows = unsigned(T) * parts;
+  if (w_dtype == kF32 && out_dtype == kF32) group_rmsnorm_kernel<float, float><<<rows, 256, 0, s>>>(x, (const float*)w, eps, (float*)out, parts, size);
+  else if (w_dtype == kF32) group_rmsnorm_kernel<float, bf16_t><<<rows, 256, 0, s>>>(x, (const float*)w, eps, (bf16_t*)out, parts, size);
+  else if (out_dtype == kF32) group_rmsnorm_kernel<bf16_t, float><<<rows, 256, 0, s>>>(x, (const bf16_t*)w, eps, (float*)out, parts, size);
+  else group_rmsnorm_kernel<bf16_t, bf16_t><<<rows, 256, 0, s>>>(x, (const bf16_t*)w, eps, (bf16_t*)out, parts, size);
+  return check_launch("sp_group_rmsnorm");
+}
+
+extern "C" int sp_activation(void* stream, int dtype, void* x, long long n, int kind) {
+  SP_REQUIRE(kind == 0, "sp_activation: no activation %d (0 = the exact GELU)", kind);
+  SP_REQUIRE((dtype == kF32 || dtype == kBF16) && n >= 0 && (x || n == 0), "sp_activation: bad arguments");
+  if (n == 0) return 0;
+  const unsigned blocks = unsigned(n / 256 + 1 < 65536 ? n / 256 + 1 : 65536);
+  if (dtype == kF32) gelu_erf_kernel<float><<<blocks, 256, 0, (hipStream_t)stream>>>((float*)x, n);
+  else gelu_erf_kernel<bf16_t><<<blocks, 256, 0, (hipStream_t)stream>>>((bf16_t*)x, n);
+  return check_launch("sp_activation");
+}
+
+extern "C" int sp_scale_rows(void* stream, int dtype, const void* x, const float* weights, int top, void* out, int T, int H) {
+  SP_REQUIRE((dtype == kF32 || dtype == kBF16) && T >= 0 && H > 0 && top > 0 && x && weights && out && x != out,
+             "sp_scale_rows: bad arguments");
+  if (T == 0) return 0;
+  const dim3 grid(unsigned(T) * top, H > 2048 ? 4 : 1);
+  if (dtype == kF32) scale_rows_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>((const float*)x, weights, top, (float*)out, H);
+  else scale_rows_kernel<bf16_t><<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)x, weights, top, (bf16_t*)out, H);
+  return check_launch("sp_scale_rows");
+}
+
+extern "C" int sp_ssd_scan(void* stream, int dtype, const void* proj, long long proj_stride, int z_off, int dt_off,
+                           const void* xbc, long long xbc_stride, int heads, int vdim, int state_size, int groups,
+                           const float* dt_bias, const float* a_log, const float* skip, const int32_t* q_start,
+                           const int32_t* q_len, const int32_t* state_slots, float* state, float* out, int T, int n_seqs) {
+  SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_ssd_scan: unsupported dtype %d", dtype);
+  SP_REQUIRE(heads > 0 && vdim > 0 && groups > 0 && heads % groups == 0 && state_size > 0 && state_size <= 256,
+             "sp_ssd_scan: %d heads of %d in %d groups with a state of %d (up to 256)", heads, vdim, groups, state_size);
+  const int inner = heads * vdim;
+  SP_REQUIRE(z_off >= 0 && dt_off >= 0 && proj_stride >= z_off + inner && proj_stride >= dt_off + heads &&
+                 xbc_stride >= inner + 2 * groups * state_size, "sp_ssd_scan: the columns do not fit the rows");
+  SP_REQUIRE(proj && xbc && dt_bias && a_log && skip && q_start && q_len && state_slots && state && out && T >= 0 && n_seqs >= 0,
+             "sp_ssd_scan: null operand");
+  if (T == 0 || n_seqs == 0) return 0;
+  const SsdArgs a = {proj, proj_stride, z_off, dt_off, xbc, xbc_stride, heads, vdim, state_size, groups, dt_bias, a_log, skip,
+                     q_start, q_len, state_slots, state, out};
+  const dim3 grid((inner + 31) / 32, n_seqs);
+  hipStream_t s = (hipStream_t)stream;
+#define SP_SSD(KPT)                                                         \
+  do {                                                                      \
+    if (dtype == kF32) ssd_scan_kernel<float, KPT><<<grid, 256, 0, s>>>(a); \
+    else ssd_scan_kernel<bf16_t, KPT><<<grid, 256, 0, s>>>(a);              \
+  } while (0)
+  if (state_size <= 32) SP_SSD(4);
+  else if (state_size <= 64) SP_SSD(8);
+  else if (state_size <= 128) SP_SSD(16);
+  else SP_SSD(32);
+#undef SP_SSD
+  return check_launch("sp_ssd_scan");
+}
+
+extern "C" int sp_selective_scan(void* stream, int dtype, const void* u, long long u_stride, int u_off, const void* z,
+                                 long long z_stride, int z_off, const float* dt, const void* bc, long long bc_stride, int bc_off,
+                                 int inner, int state_size, const float* a, const float* skip, const int32_t* q_start,
+                                 const int32_t* q_len, const int32_t* state_slots, float* state, void* out, int T, int n_seqs) {
+  SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_selective_scan: unsupported dtype %d", dtype);
+  SP_REQUIRE(inner > 0 && state_size > 0 && state_size <= 256, "sp_selective_scan: %d channels with a state of %d (up to 256)",
+             inner, state_size);
+  SP_REQUIRE(u_off >= 0 && z_off >= 0 && bc_off >= 0 && u_stride >= u_off + inner && z_stride >= z_off + inner &&
+                 bc_stride >= bc_off + 2 * state_size, "sp_selective_scan: the columns do not fit the rows");
+  SP_REQUIRE(u && z && dt && bc && a && skip && q_start && q_len && state_slots && state && out && T >= 0 && n_seqs >= 0,
+             "sp_selective_scan: null operand");
+  if (T == 0 || n_seqs == 0) return 0;
+  const SelArgs args = {u, u_stride, u_off, z, z_stride, z_off, dt, bc, bc_stride, bc_off, inner, state_size, a, skip,
+                        q_start, q_len, state_slots, state, out};
+  const dim3 grid((inner + 63) / 64, n_seqs);
+  hipStream_t s = (hipStream_t)stream;
+#define SP_SEL(KPT)                                                                  \
+  do {                                                                               \
+    if (dtype == kF32) selective_scan_kernel<float, KPT><<<grid, 256, 0, s>>>(args); \
+    else selective_scan_kernel<bf16_t, KPT><<<grid, 256, 0, s>>>(args);              \
+  } while (0)
+  if (state_size <= 16) SP_SEL(4);
+  else if (state_size <= 32) SP_SEL(8);
+  else if (state_size <= 64) SP_SEL(16);
+  else if (state_size <= 128) SP_SEL(32);
+  else SP_SEL(64);
+#undef SP_SEL
+  return check_launch("sp_selective_scan");
+}
+
+extern "C" int sp_qk_cross_prepare(void* stream, int dtype, const void* qk, int nq, int nkv, int dim, int width, int w_dtype,
+                                   const void* q_norm, const void* k_norm, float eps, const int32_t* positions,
+                                   const double* freq, int rotary_dim, const int32_t* slot_mapping, void* q_out, void* k_pool,
+                                   void* v_pool, int page_size, int T) {
+  SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_qk_cross_prepare: unsupported dtype %d", dtype);
+  SP_REQUIRE(w_dtype == dtype || w_dtype == kF32, "sp_qk_cross_prepare: norm weights of dtype %d beside rows of dtype %d", w_dtype, dtype);
+  SP_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0 && dim > 0 && width >= dim && dim <= 4096,
+             "sp_qk_cross_prepare: %d heads over %d of %d numbers at width %d", nq, nkv, dim, width);
+  SP_REQUIRE(rotary_dim >= 0 && rotary_dim % 2 == 0 && rotary_dim <= dim && (rotary_dim == 0 || freq),
+             "sp_qk_cross_prepare: %d of %d numbers cannot turn in pairs", rotary_dim, dim);
+  SP_REQUIRE(qk && q_norm && k_norm && positions && q_out && (!slot_mapping || (k_pool && v_pool && page_size > 0)) && T >= 0,
+             "sp_qk_cross_prepare: null operand");
+  if (T == 0) return 0;
+  const CrossArgs a = {qk, nq, nkv, dim, width, q_norm, k_norm, eps, positions, freq, rotary_dim, slot_mapping, q_out,
+                       k_pool, v_pool, page_size};
+  const dim3 grid(T, nq + nkv);
+  const size_t lds = sizeof(float) * (2 * size_t(dim) + 16);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == kF32) qk_cross_prepare_kernel<float, float, true><<<grid, 128, lds, s>>>(a);
+  else if (w_dtype == kF32) qk_cross_prepare_kernel<bf16_t, float, false><<<grid, 128, lds, s>>>(a);
+  else qk_cross_prepare_kernel<bf16_t, bf16_t, false><<<grid, 128, lds, s>>>(a);
+  return check_launch("sp_qk_cross_prepare");
+}
+
+extern "C" int sp_head_mix(void* stream, int dtype, const void* o, const float* talk, int nq, int nkv, int dim, int width,
+                           void* out, int T) {
+  SP_REQUIRE((dtype == kF32 || dtype == kBF16) && nq > 0 && nkv > 0 && nq % nkv == 0 && dim > 0 && width >= dim && T >= 0 && o &&
+                 talk && out && o != out, "sp_head_mix: bad arguments");
+  if (T == 0) return 0;
+  const dim3 grid(T, nq);
+  if (dtype == kF32) head_mix_kernel<float><<<grid, 128, 0, (hipStream_t)stream>>>((const float*)o, talk, nq, nkv, dim, width, (float*)out);
+  else head_mix_kernel<bf16_t><<<grid, 128, 0, (hipStream_t)stream>>>((const bf16_t*)o, talk, nq, nkv, dim, width, (bf16_t*)out);
+  return check_launch("sp_head_mix");
+}

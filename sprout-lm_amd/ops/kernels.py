@@ -267,6 +267,22 @@ def route(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, row_of
                              row_of_pair.data_ptr(), pair_of_row.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr()))
 
 
+def route_sigmoid(logits: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, row_of_pair, pair_of_row, tiles, n_tiles,
+                  tile_rows: int = 64) -> None:
+    """`route` whose weights are the sigmoid of each chosen logit, not renormalised."""
+    _gpu(logits, "router logits"); _gpu(ids, "chosen experts"); _gpu(weights, "expert weights")
+    T, E = logits.shape
+    top = ids.shape[1]
+    if logits.dtype != torch.float32 or ids.dtype != torch.int32 or weights.dtype != torch.float32 or \
+            tuple(ids.shape) != (T, top) or tuple(weights.shape) != (T, top) or not 0 < top <= E:
+        raise KernelError("route_sigmoid: float32 logits [T, E], int32 ids and float32 weights [T, top] expected")
+    pairs = T * top
+    _ints(row_of_pair, pairs, "row_of_pair"); _ints(pair_of_row, pairs, "pair_of_row")
+    _ints(tiles, 3 * route_max_tiles(pairs, E, tile_rows), "expert tiles"); _ints(n_tiles, 1, "tile count")
+    check(library().sp_route_sigmoid(_stream(), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), T, E, top, tile_rows,
+                                     row_of_pair.data_ptr(), pair_of_row.data_ptr(), tiles.data_ptr(), n_tiles.data_ptr()))
+
+
 def route_sort(ids: torch.Tensor, experts: int, row_of_pair, pair_of_row, tiles, n_tiles, tile_rows: int = 64) -> None:
     """Orders the (token, choice) pairs by expert for the grouped products (see sprout_hip.h)."""
     pairs = ids.numel()
@@ -305,8 +321,9 @@ def expert_down(act: torch.Tensor, w: torch.Tensor, tiles, n_tiles, out: torch.T
                                    n_tiles.data_ptr(), max_tiles, tile_rows, out.data_ptr(), rows, E, hidden, inner))
 
 
-def route_combine(y: torch.Tensor, row_of_pair, weights: torch.Tensor, residual: torch.Tensor) -> None:
-    """residual[t] += sum_k weights[t, k] * y[row_of_pair[t * top + k]]."""
+def route_combine(y: torch.Tensor, row_of_pair, weights: torch.Tensor, residual: torch.Tensor, weighted: bool = True) -> None:
+    """residual[t] += sum_k weights[t, k] * y[row_of_pair[t * top + k]]; with `weighted` False the rows are added as
+    they are (`weights` then only says how many choices a token has)."""
     _gpu(y, "expert outputs"); _gpu(weights, "expert weights"); _gpu(residual, "residual")
     T, top = weights.shape
     H = residual.shape[1]
@@ -314,8 +331,8 @@ def route_combine(y: torch.Tensor, row_of_pair, weights: torch.Tensor, residual:
             or weights.dtype != torch.float32:
         raise KernelError("route_combine: float32 outputs [T * top, H], weights [T, top] and residual [T, H] expected")
     _ints(row_of_pair, T * top, "row_of_pair")
-    check(library().sp_route_combine(_stream(), y.data_ptr(), row_of_pair.data_ptr(), weights.data_ptr(), top,
-                                     residual.data_ptr(), T, H))
+    check(library().sp_route_combine(_stream(), y.data_ptr(), row_of_pair.data_ptr(), weights.data_ptr() if weighted else None,
+                                     top, residual.data_ptr(), T, H))
 
 
 def route_scored(logits: torch.Tensor, outputs: int, real: int, correction, groups: int, keep: int, scale: float,
@@ -523,13 +540,15 @@ def attention_plan(dtype: torch.dtype, hd: int, page_size: int, nq: int, nkv: in
 def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torch.Tensor, block_tables: torch.Tensor,
               batch: AttentionBatch, out: torch.Tensor, nq: int, nkv: int, hd: int, window: int | None, scale: float,
               workspace=None, kind: int = 0, project=None, scores: str = "scaled_dot", softcap: float = 0.0,
-              sinks: torch.Tensor | None = None, mask_chunk: int | None = None) -> bool:
+              sinks: torch.Tensor | None = None, mask_chunk: int | None = None, keep_first: int = 0) -> bool:
     """Causal attention of a mixed batch over paged keys and values (see sprout_hip.h).
 
     `workspace(n)` must return a float32 device tensor of at least n elements (default: a new one).
     `scores`: "scaled_dot", or "capped" (the scaled product s becomes softcap * tanh(s / softcap)).  `sinks`: float32
     [nq], one logit per query head that joins the softmax's denominator without a key or value.  `mask_chunk`: a
     query sees only the keys of its own block of that many positions, counted from position 0.
+    `keep_first`: a sequence's first keep_first keys stay visible to every later query beside its `window`; the
+    float32-arithmetic kernel on the vector units is the one that knows them, and such a call runs on it.
     `project`: (w_o [hidden, nq * hd], residual float32 [T, hidden]) of an output projection without bias
     that may be folded in: where the kernels take the step that way (one-query sequences only, bfloat16),
     residual += attention . w_o^T, `out` is left untouched and True is returned; otherwise False, and the
@@ -543,6 +562,11 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
         if sinks.dtype != torch.float32 or sinks.numel() != nq:
             raise KernelError(f"attention: sinks must be {nq} float32 values")
     stage = (float(softcap), _ptr(sinks), int(mask_chunk) if mask_chunk else 0)
+    keep_first = int(keep_first) if window else 0      # without a window every earlier key is visible anyway
+    if keep_first < 0 or (keep_first and mask_chunk):
+        raise KernelError("attention: kept first keys go with a window alone, and their number is not negative")
+    if keep_first:
+        kind = 2
     for t, what in ((q, "q"), (out, "attention output")):
         _gpu(t, what)
     T = out.shape[0]
@@ -610,7 +634,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
                                  _ptr(decode) if n_decode and decode is not None else None, n_decode,
                                  max_decode_ctx, _ptr(ws),
                                  need, out.data_ptr(), nq, nkv, hd, page_size, num_pages, int(window) if window else 0,
-                                 float(scale), kind, scores_code, *stage))
+                                 float(scale), kind, scores_code, *stage, keep_first))
     return False
 
 
@@ -805,6 +829,159 @@ def rglru(proj: torch.Tensor, y_off: int, x_off: int, width: int, blocks: int, t
                              lam.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), seq_of_token.data_ptr(), state_slots.data_ptr(),
                              state.data_ptr(), _ptr(tail) if taps > 1 else None, decay.data_ptr(), drive.data_ptr(),
                              out.data_ptr(), T, n_seqs, int(max_q_len) if carry is not None else 0, _ptr(carry)))
+
+
+def _step_ints(q_start, q_len, state_slots, n_seqs: int, seq_of_token=None, T: int = 0) -> None:
+    for t, what in ((q_start, "q_start"), (q_len, "q_len"), (state_slots, "state_slots")):
+        _ints(t, n_seqs, what)
+    if seq_of_token is not None:
+        _ints(seq_of_token, T, "seq_of_token")
+
+
+def short_conv(x: torch.Tensor, x_off: int, channels: int, taps: int, w: torch.Tensor, bias, out: torch.Tensor, out_off: int,
+               q_start, q_len, seq_of_token, state_slots, n_seqs: int, state, act: str | None = None,
+               add_input: bool = False) -> None:
+    """The causal convolution of sp_short_conv (sprout_hip.h) on columns x_off .. x_off + channels of a step's rows `x`, into
+    columns out_off .. of `out` (another tensor of the same dtype).  `state`: float32 [slots, taps - 1, channels], the
+    requests' last inputs, read and left behind; None with one tap.  `act`: None or "silu"."""
+    _gpu(x, "convolution input"); _gpu(out, "convolution output"); _gpu(w, "convolution weights")
+    T = out.shape[0]
+    if x.dim() != 2 or out.dim() != 2 or x.shape[0] < T or x.dtype != out.dtype or x_off + channels > x.shape[1] \
+            or out_off + channels > out.shape[1] or x.data_ptr() == out.data_ptr():
+        raise KernelError(f"short_conv: rows {tuple(x.shape)} {x.dtype} and {tuple(out.shape)} {out.dtype} do not fit {channels} channels")
+    if tuple(w.shape) != (channels, taps) or not w.is_contiguous() or (bias is not None and (bias.numel() != channels or bias.dtype != w.dtype)):
+        raise KernelError(f"short_conv: weights must be [{channels}, {taps}] with a bias of {channels}")
+    if act not in (None, "silu"):
+        raise KernelError(f"short_conv: no activation {act!r}")
+    _step_ints(q_start, q_len, state_slots, n_seqs, seq_of_token, T)
+    if taps > 1:
+        _gpu(state, "convolution state")
+        if state.dtype != torch.float32 or state.dim() != 3 or tuple(state.shape[1:]) != (taps - 1, channels) or not state.is_contiguous():
+            raise KernelError(f"short_conv: the state must be float32 [slots, {taps - 1}, {channels}]")
+    if bias is not None:
+        _gpu(bias, "convolution bias")
+    check(library().sp_short_conv(_stream(), _code(x, "convolution input"), x.data_ptr(), x.stride(0), x_off, channels, taps,
+                                  _code(w, "convolution weights"), w.data_ptr(), _ptr(bias), 1 if act == "silu" else 0,
+                                  int(bool(add_input)), out.data_ptr(), out.stride(0), out_off, q_start.data_ptr(),
+                                  q_len.data_ptr(), seq_of_token.data_ptr(), state_slots.data_ptr(),
+                                  state.data_ptr() if taps > 1 else None, T, n_seqs))
+
+
+def group_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, parts: int) -> None:
+    """out = x / sqrt(mean(x^2) + eps) * weight with the mean over each of a row's `parts` equal parts; x float32 [T, n]."""
+    _gpu(x, "norm input"); _gpu(weight, "norm weight"); _gpu(out, "norm output")
+    T, n = out.shape
+    if x.dtype != torch.float32 or tuple(x.shape) != (T, n) or weight.numel() != n or parts <= 0 or n % parts \
+            or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError(f"group_rmsnorm: float32 rows {tuple(x.shape)}, weight {tuple(weight.shape)} and {parts} parts do not fit")
+    check(library().sp_group_rmsnorm(_stream(), x.data_ptr(), _code(weight, "norm weight"), weight.data_ptr(), float(eps),
+                                     _code(out, "norm output"), out.data_ptr(), T, parts, n // parts))
+
+
+UNARY_ACTIVATIONS = {"gelu_erf": 0}      # x * Phi(x), the exact GELU
+
+
+def activation(x: torch.Tensor, kind: str) -> None:
+    """In place: x <- act(x), `kind` one of UNARY_ACTIVATIONS."""
+    _gpu(x, "activation input")
+    if not x.is_contiguous():
+        raise KernelError("activation: rows must be contiguous")
+    check(library().sp_activation(_stream(), _code(x, "activation input"), x.data_ptr(), x.numel(),
+                                  variant_code(UNARY_ACTIVATIONS, kind, "activation")))
+
+
+def scale_rows(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t * top + k] = x[t] * weights[t, k]: a token's row once per choice, times the choice's weight."""
+    _gpu(x, "rows"); _gpu(weights, "row weights"); _gpu(out, "scaled rows")
+    T, top = weights.shape
+    H = x.shape[1]
+    if weights.dtype != torch.float32 or x.shape[0] < T or tuple(out.shape) != (T * top, H) or out.dtype != x.dtype \
+            or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError("scale_rows: rows [T, H], float32 weights [T, top] and an output [T * top, H] of the rows' dtype expected")
+    check(library().sp_scale_rows(_stream(), _code(x, "rows"), x.data_ptr(), weights.data_ptr(), top, out.data_ptr(), T, H))
+
+
+def ssd_scan(proj: torch.Tensor, z_off: int, dt_off: int, xbc: torch.Tensor, heads: int, vdim: int, state_size: int, groups: int,
+             dt_bias, a_log, skip, q_start, q_len, state_slots, n_seqs: int, state: torch.Tensor, out: torch.Tensor) -> None:
+    """The state-space-duality scan of sp_ssd_scan (sprout_hip.h); out float32 [T, heads * vdim] = y * silu(z)."""
+    for t, what in ((proj, "projections"), (xbc, "convolved rows"), (state, "state"), (out, "scan output")):
+        _gpu(t, what)
+    T, inner = out.shape[0], heads * vdim
+    if proj.shape[0] < T or xbc.shape[0] < T or proj.dtype != xbc.dtype or out.dtype != torch.float32 or tuple(out.shape) != (T, inner) \
+            or not out.is_contiguous():
+        raise KernelError("ssd_scan: rows and output do not fit")
+    for t in (dt_bias, a_log, skip):
+        _gpu(t, "head constants")
+        if t.dtype != torch.float32 or t.numel() != heads:
+            raise KernelError(f"ssd_scan: one float32 constant per head ({heads}) expected")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, state_size, vdim) or not state.is_contiguous():
+        raise KernelError(f"ssd_scan: the state must be float32 [slots, {heads}, {state_size}, {vdim}]")
+    _step_ints(q_start, q_len, state_slots, n_seqs)
+    check(library().sp_ssd_scan(_stream(), _code(proj, "projections"), proj.data_ptr(), proj.stride(0), z_off, dt_off,
+                                xbc.data_ptr(), xbc.stride(0), heads, vdim, state_size, groups, dt_bias.data_ptr(),
+                                a_log.data_ptr(), skip.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), state_slots.data_ptr(),
+                                state.data_ptr(), out.data_ptr(), T, n_seqs))
+
+
+def selective_scan(u: torch.Tensor, u_off: int, z: torch.Tensor, z_off: int, dt: torch.Tensor, bc: torch.Tensor, bc_off: int,
+                   inner: int, state_size: int, a, skip, q_start, q_len, state_slots, n_seqs: int, state: torch.Tensor,
+                   out: torch.Tensor) -> None:
+    """The selective scan of sp_selective_scan (sprout_hip.h); out [T, inner] of the rows' dtype = y * silu(z)."""
+    for t, what in ((u, "inputs"), (z, "gates"), (dt, "step sizes"), (bc, "B and C"), (state, "state"), (out, "scan output")):
+        _gpu(t, what)
+    T = out.shape[0]
+    if min(u.shape[0], z.shape[0], dt.shape[0], bc.shape[0]) < T or not (u.dtype == z.dtype == bc.dtype == out.dtype) \
+            or dt.dtype != torch.float32 or tuple(dt.shape[1:]) != (inner,) or tuple(out.shape) != (T, inner) \
+            or not dt.is_contiguous() or not out.is_contiguous():
+        raise KernelError("selective_scan: rows and output do not fit")
+    _gpu(a, "decay rates"); _gpu(skip, "skip weights")
+    if a.dtype != torch.float32 or tuple(a.shape) != (inner, state_size) or skip.dtype != torch.float32 or skip.numel() != inner:
+        raise KernelError(f"selective_scan: float32 rates [{inner}, {state_size}] and skips [{inner}] expected")
+    if state.dtype != torch.float32 or tuple(state.shape[1:]) != (inner, state_size) or not state.is_contiguous():
+        raise KernelError(f"selective_scan: the state must be float32 [slots, {inner}, {state_size}]")
+    _step_ints(q_start, q_len, state_slots, n_seqs)
+    check(library().sp_selective_scan(_stream(), _code(u, "inputs"), u.data_ptr(), u.stride(0), u_off, z.data_ptr(), z.stride(0),
+                                      z_off, dt.data_ptr(), bc.data_ptr(), bc.stride(0), bc_off, inner, state_size, a.data_ptr(),
+                                      skip.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), state_slots.data_ptr(),
+                                      state.data_ptr(), out.data_ptr(), T, n_seqs))
+
+
+def qk_cross_prepare(qk: torch.Tensor, nq: int, nkv: int, dim: int, width: int, q_norm, k_norm, eps: float, positions, freq,
+                     rotary_dim: int, q_out: torch.Tensor, slot_mapping=None, k_pool=None, v_pool=None) -> None:
+    """sp_qk_cross_prepare (sprout_hip.h): head norms, turning in neighbouring pairs, and the (query head, value head)
+    pairs as heads of their own: queries to q_out [T, nq * nkv * width], keys and values into pools of nkv * nkv heads."""
+    _gpu(qk, "q and k rows"); _gpu(q_out, "prepared queries"); _gpu(q_norm, "q norm"); _gpu(k_norm, "k norm")
+    T = q_out.shape[0]
+    if qk.shape[0] < T or qk.shape[1] != (nq + nkv) * dim or not qk.is_contiguous() or q_out.dtype != qk.dtype \
+            or tuple(q_out.shape) != (T, nq * nkv * width) or not q_out.is_contiguous():
+        raise KernelError(f"qk_cross_prepare: rows {tuple(qk.shape)} and queries {tuple(q_out.shape)} do not fit")
+    if q_norm.numel() != dim or k_norm.numel() != dim or q_norm.dtype != k_norm.dtype:
+        raise KernelError(f"qk_cross_prepare: norm weights of {dim} numbers expected")
+    _ints(positions, T, "positions")
+    if rotary_dim:
+        _gpu(freq, "frequencies")
+        if freq.dtype != torch.float64 or freq.numel() < rotary_dim // 2:
+            raise KernelError("qk_cross_prepare: a float64 table of one frequency per pair expected")
+    page_size = 0
+    if slot_mapping is not None:
+        _ints(slot_mapping, T, "slot_mapping")
+        _, page_size = _check_pools(k_pool, v_pool, nkv * nkv, width, qk.dtype, "qk_cross_prepare")
+    check(library().sp_qk_cross_prepare(_stream(), _code(qk, "q and k rows"), qk.data_ptr(), nq, nkv, dim, width,
+                                        _code(q_norm, "q norm"), q_norm.data_ptr(), k_norm.data_ptr(), float(eps),
+                                        positions.data_ptr(), _ptr(freq) if rotary_dim else None, rotary_dim, _ptr(slot_mapping),
+                                        q_out.data_ptr(), _ptr(k_pool), _ptr(v_pool), page_size, T))
+
+
+def head_mix(o: torch.Tensor, talk: torch.Tensor, nq: int, nkv: int, dim: int, width: int, out: torch.Tensor) -> None:
+    """sp_head_mix (sprout_hip.h): the outputs of the (query head, value head) heads mixed by `talk` float32 [nq, nq]."""
+    _gpu(o, "attention outputs"); _gpu(talk, "head mixing matrix"); _gpu(out, "mixed heads")
+    T = out.shape[0]
+    if o.shape[0] < T or o.shape[1] != nq * nkv * width or not o.is_contiguous() or out.dtype != o.dtype \
+            or tuple(out.shape) != (T, nq * dim) or not out.is_contiguous() or talk.dtype != torch.float32 \
+            or tuple(talk.shape) != (nq, nq) or not talk.is_contiguous():
+        raise KernelError("head_mix: outputs, matrix and result do not fit")
+    check(library().sp_head_mix(_stream(), _code(o, "attention outputs"), o.data_ptr(), talk.data_ptr(), nq, nkv, dim, width,
+                                out.data_ptr(), T))
 
 
 def retention_takes(dim: int, vdim: int) -> bool:

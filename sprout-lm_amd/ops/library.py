@@ -24,7 +24,7 @@ def _declare(lib):
                           c_int, c_int, c_int, c_int, c_int],
         "sp_attention": [c_void, c_int, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_void,
                          c_int, c_int, c_int, c_int, c_void, c_int, c_int, c_void, c_i64, c_void, c_int, c_int, c_int, c_int,
-                         c_int, c_int, c_float, c_int, c_int, c_float, c_void, c_int],
+                         c_int, c_int, c_float, c_int, c_int, c_float, c_void, c_int, c_int],
         "sp_attention_decode_project_takes": [c_int] * 7,
         "sp_attention_decode_project": [c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void,
                                         c_int, c_int, c_void, c_i64, c_void, c_void, c_int, c_int, c_int, c_int, c_int,
@@ -80,6 +80,19 @@ def _declare(lib):
                            c_float, c_int],
         "sp_expert_down": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_void, c_int, c_int, c_int, c_int],
         "sp_route_combine": [c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_int],
+        "sp_route_sigmoid": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void, c_void, c_void, c_void],
+        "sp_short_conv": [c_void, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_void, c_void, c_int, c_int, c_void, c_i64,
+                          c_int, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
+        "sp_group_rmsnorm": [c_void, c_void, c_int, c_void, c_float, c_int, c_void, c_int, c_int, c_int],
+        "sp_activation": [c_void, c_int, c_void, c_i64, c_int],
+        "sp_scale_rows": [c_void, c_int, c_void, c_void, c_int, c_void, c_int, c_int],
+        "sp_ssd_scan": [c_void, c_int, c_void, c_i64, c_int, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_void, c_void,
+                        c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
+        "sp_selective_scan": [c_void, c_int, c_void, c_i64, c_int, c_void, c_i64, c_int, c_void, c_void, c_i64, c_int, c_int,
+                              c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
+        "sp_qk_cross_prepare": [c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_int, c_void, c_void, c_float, c_void,
+                                c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int],
+        "sp_head_mix": [c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_void, c_int],
         "sp_probe_read": [c_void, c_void, c_i64, c_int, c_void],
         "sp_probe_mfma": [c_void, c_int, c_int, c_void, ctypes.POINTER(ctypes.c_double)],
     }

@@ -12,7 +12,7 @@ from typing import Callable
 from ..weights.loader import TensorSpec
 
 _REGISTRIES: dict[str, dict[str, type]] = {
-    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "embedding": {}, "head": {}, "scale": {},
+    "mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {}, "embedding": {}, "head": {}, "scale": {}, "conv": {},
 }
 
 

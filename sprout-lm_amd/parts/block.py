@@ -7,17 +7,20 @@ from .base import Block, register_part
 @register_part("block", "pre_norm")
 class PreNormBlock(Block):
     """x += mixer(norm(x)); x += feed_forward(norm(x)).  The residual stream x is float32.  `ffn` (and its norm) may
-    be absent: the layer is then its mixer alone."""
+    be absent: the layer is then its mixer alone.  `mixer_conv`: a part that stands between the norm and the mixer (a
+    short convolution over time, which keeps its last inputs per request): the mixer reads mixer_conv(norm(x))."""
 
     graph_safe = True
 
     graph_safe_portions = True
 
-    def __init__(self, mixer_norm, mixer, ffn_norm=None, ffn=None):
-        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn = mixer_norm, mixer, ffn_norm, ffn
+    def __init__(self, mixer_norm, mixer, ffn_norm=None, ffn=None, mixer_conv=None):
+        self.mixer_norm, self.mixer, self.ffn_norm, self.ffn, self.mixer_conv = mixer_norm, mixer, ffn_norm, ffn, mixer_conv
 
     def parts(self):
         named = {"mixer_norm": self.mixer_norm, "mixer": self.mixer}
+        if self.mixer_conv is not None:
+            named["mixer_conv"] = self.mixer_conv
         if self.ffn is not None:
             named.update({"ffn_norm": self.ffn_norm, "ffn": self.ffn})
         return named
@@ -26,7 +29,12 @@ class PreNormBlock(Block):
         T, H = residual.shape
         cache = caches.get("mixer")
         h = ctx.buffer("normed", (T, H), ctx.act_dtype)
-        if not self.mixer.forward_from_residual(ctx, self.mixer_norm, residual, cache):
+        if self.mixer_conv is not None:
+            self.mixer_norm.forward(ctx, residual, h)
+            mixed_in = ctx.buffer("normed_conv", (T, H), ctx.act_dtype)
+            self.mixer_conv.forward(ctx, h, mixed_in, caches.get("mixer_conv"))
+            self.mixer.forward(ctx, mixed_in, residual, cache)
+        elif not self.mixer.forward_from_residual(ctx, self.mixer_norm, residual, cache):
             self.mixer_norm.forward(ctx, residual, h)
             self.mixer.forward(ctx, h, residual, cache)
         if self.ffn is None:

@@ -8,17 +8,21 @@ from .base import Part, register_part
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Part):
+    """x = table[token] * scale, float32."""
+
     graph_safe = True
     graph_safe_portions = True
 
-    def __init__(self, vocab: int, hidden: int, tensor: str = "weight"):
-        self.vocab, self.hidden, self.tensor = vocab, hidden, tensor
+    def __init__(self, vocab: int, hidden: int, tensor: str = "weight", scale: float = 1.0):
+        self.vocab, self.hidden, self.tensor, self.scale = vocab, hidden, tensor, float(scale)
 
     def tensors(self):
         return {self.tensor: TensorSpec((self.vocab, self.hidden))}
 
     def forward(self, ctx, tokens, residual):
         ops.embed(self.w[self.tensor], tokens, residual)
+        if self.scale != 1.0:
+            ops.scale(residual, self.scale)
 
     def weight_elements(self) -> int:
         return 0      # a step gathers one row per token: nothing beside the matrices

@@ -91,3 +91,46 @@ class GatedMLP(FeedForward):
             ops.silu_mul(gu, act, activation=self.activation, limit=self.limit, row_gate=row_gate,
                          row_gate_column=row_gate_column)
         ops.gemm(act, self.w_down, residual, accumulate=True)
+
+
+@register_part("feed_forward", "mlp")
+class DenseMLP(FeedForward):
+    """down(act(up(x) + b_up)) + b_down, no gate.  `activation`: one of `ops.UNARY_ACTIVATIONS` ("gelu_erf": the exact
+    GELU, x * Phi(x)).  `bias`: the suffix of the biases' names, None for projections without them.  `tensors`: local
+    names of the up and down matrices."""
+
+    graph_safe = True
+
+    graph_safe_portions = True
+
+    def __init__(self, hidden: int, inner: int, activation: str = "gelu_erf", bias: str | None = ".b",
+                 tensors: tuple = ("up", "down")):
+        if activation not in ops.UNARY_ACTIVATIONS:
+            raise ValueError(f"Feed-forward with activation {activation!r} has no kernel; there are kernels for "
+                             f"{sorted(ops.UNARY_ACTIVATIONS)}.")
+        self.hidden, self.inner, self.activation, self.bias = hidden, inner, activation, bias
+        self.names = tuple(tensors)
+
+    def flops(self, tokens: int, pairs: int = 0) -> float:
+        return 2.0 * tokens * 2 * self.hidden * self.inner
+
+    def tensors(self):
+        up, down = self.names
+        out = {up: TensorSpec((self.inner, self.hidden)), down: TensorSpec((self.hidden, self.inner))}
+        if self.bias is not None:
+            out.update({up + self.bias: TensorSpec((self.inner,), "vector"), down + self.bias: TensorSpec((self.hidden,), "vector")})
+        return out
+
+    def bind(self, tensors):
+        up, down = self.names
+        self.w_up, self.w_down = tensors[up], tensors[down]
+        self.b_up = tensors[up + self.bias] if self.bias is not None else None
+        self.b_down = tensors[down + self.bias] if self.bias is not None else None
+        self.w = {}
+
+    def forward(self, ctx, h, residual):
+        T = h.shape[0]
+        act = ctx.buffer("mlp_inner", (T, self.inner), ctx.act_dtype)
+        ops.gemm(h, self.w_up, act, bias=self.b_up)
+        ops.activation(act, self.activation)
+        ops.gemm(act, self.w_down, residual, bias=self.b_down, accumulate=True)

@@ -29,6 +29,9 @@ class RoutedExperts(FeedForward):
     s + correction (a tensor, `correction`) and only among the outputs of the `keep` best of `groups` equal groups of
     neighbours (a group's worth is its largest such sum); the weights are the chosen outputs' s times `route_scale`, not
     renormalised.  The last `identity` router outputs are experts without tensors that return their input.
+    routing "sigmoid_top": the `top` largest logits are chosen and a choice's weight is the sigmoid of its logit, not
+    renormalised.  weight_on "input": the weight multiplies what the expert reads, not what it returns: the output is the
+    sum of expert_e(weight_e * x).
     activation / limit, shared_activation / shared_limit: see GatedMLP.  shared_gate: the local name of a [1, hidden]
     tensor g; the shared expert's output is then multiplied by sigmoid(g . x), one number per token.
     """
@@ -42,14 +45,16 @@ class RoutedExperts(FeedForward):
                  tensors: tuple = ("e{e}.gate", "e{e}.up", "e{e}.down", "router", "router.b", "shared."),
                  limit: float = 0.0, routing: str = "softmax_top", identity: int = 0, groups: int = 1, keep: int = 1,
                  route_scale: float = 1.0, correction: str | None = None, shared_activation: str | None = None,
-                 shared_limit: float = 0.0, shared_gate: str | None = None):
+                 shared_limit: float = 0.0, shared_gate: str | None = None, weight_on: str = "output"):
         if min(hidden, inner, experts, top) <= 0 or top > experts + identity or identity < 0:
             raise ConfigError(f"A routed feed-forward needs 0 < top <= experts and positive sizes, got top={top} "
                               f"experts={experts} inner={inner}.")
-        if routing not in ("softmax_top", "scored_groups"):
-            raise ConfigError(f"No routing rule {routing!r}; there are 'softmax_top' and 'scored_groups'.")
+        if routing not in ("softmax_top", "scored_groups", "sigmoid_top"):
+            raise ConfigError(f"No routing rule {routing!r}; there are 'softmax_top', 'sigmoid_top' and 'scored_groups'.")
+        if weight_on not in ("output", "input") or (weight_on == "input" and identity):
+            raise ConfigError(f"A choice's weight goes on the expert's 'output' or its 'input' (then without identity experts), got {weight_on!r}.")
         outputs = experts + identity
-        if routing == "softmax_top" and (identity or groups != 1 or correction or route_scale != 1.0):
+        if routing != "scored_groups" and (identity or groups != 1 or correction or route_scale != 1.0):
             raise ConfigError("Identity experts, groups, a correction and a scale belong to the rule 'scored_groups'.")
         if routing == "scored_groups":
             if groups <= 0 or outputs % groups or not 0 < keep <= groups or top > keep * (outputs // groups):
@@ -67,7 +72,7 @@ class RoutedExperts(FeedForward):
         self.router_bias, self.activation, self.names = router_bias, activation, tuple(tensors)
         self.limit, self.routing, self.identity, self.groups, self.keep = float(limit), routing, identity, groups, keep
         self.route_scale, self.correction, self.shared_gate = float(route_scale), correction, shared_gate
-        self.outputs = outputs
+        self.outputs, self.weight_on = outputs, weight_on
         prefix = self.names[5]
         try:
             self.shared = None if not shared_inner else GatedMLP(hidden, shared_inner, shared_activation or activation,
@@ -134,17 +139,25 @@ class RoutedExperts(FeedForward):
         if self.routing == "scored_groups":
             ops.route_scored(logits, self.outputs, E, self.w_correction, self.groups, self.keep, self.route_scale, ids, weights,
                              row_of_pair, pair_of_row, tiles, n_tiles, tile_rows)
+        elif self.routing == "sigmoid_top":
+            ops.route_sigmoid(logits, ids, weights, row_of_pair, pair_of_row, tiles, n_tiles, tile_rows)
         else:
             ops.route(logits, ids, weights, row_of_pair, pair_of_row, tiles, n_tiles, tile_rows)
         act = ctx.buffer("expert_act", (pairs, self.inner), ctx.act_dtype)
-        ops.expert_gate_up(h, self.w_gate_up, tiles, n_tiles, pair_of_row, top, act, activation=self.activation,
-                           tile_rows=tile_rows, limit=self.limit)
+        if self.weight_on == "input":      # every (token, choice) pair reads a row of its own: the token's, times the weight
+            scaled = ctx.buffer("expert_in", (pairs, self.hidden), ctx.act_dtype)
+            ops.scale_rows(h, weights, scaled)
+            ops.expert_gate_up(scaled, self.w_gate_up, tiles, n_tiles, pair_of_row, 1, act, activation=self.activation,
+                               tile_rows=tile_rows, limit=self.limit)
+        else:
+            ops.expert_gate_up(h, self.w_gate_up, tiles, n_tiles, pair_of_row, top, act, activation=self.activation,
+                               tile_rows=tile_rows, limit=self.limit)
         out = ctx.buffer("expert_out", (pairs, self.hidden), torch.float32)
         ops.expert_down(act, self.w_down, tiles, n_tiles, out, tile_rows=tile_rows)
         if self.identity:      # a pair routed to an identity output has no row of `out`: the sum takes the token's input
             ops.route_combine_identity(out, row_of_pair, ids, weights, h, E, residual)
         else:
-            ops.route_combine(out, row_of_pair, weights, residual)
+            ops.route_combine(out, row_of_pair, weights, residual, weighted=self.weight_on == "output")
         if self.shared is not None:
             if self.shared_gate is not None:
                 self.shared.forward(ctx, h, residual, row_gate=logits, row_gate_column=self.outputs)

@@ -9,24 +9,32 @@ from .base import Norm, NormFold, register_part
 @register_part("norm", "rmsnorm")
 class RMSNorm(Norm):
     """y = x / sqrt(mean(x^2) + eps) * weight; sums in float32, the weight is used as it is.  `tensor`: the local
-    name of the weight."""
+    name of the weight.  `one_plus`: the tensor holds the weight's distance from one, y = ... * (1 + tensor); the sum
+    1 + tensor is taken once, in float32, when the tensor is bound."""
 
     graph_safe = True
 
     graph_safe_portions = True
 
-    def __init__(self, size: int, eps: float, tensor: str = "weight"):
-        self.size, self.eps, self.tensor = size, eps, tensor
+    def __init__(self, size: int, eps: float, tensor: str = "weight", one_plus: bool = False):
+        self.size, self.eps, self.tensor, self.one_plus = size, eps, tensor, bool(one_plus)
 
     def tensors(self):
-        return {self.tensor: TensorSpec((self.size,), "vector", "one_plus_normal")}
+        return {self.tensor: TensorSpec((self.size,), "vector", "normal" if self.one_plus else "one_plus_normal")}
+
+    def bind(self, tensors):
+        self.w = tensors
+        self.weight = tensors[self.tensor]
+        if self.one_plus:
+            import torch
+            self.weight = (tensors[self.tensor].to(torch.float32) + 1.0).contiguous()
 
     def forward(self, ctx, x, out, rows=None):
-        ops.rmsnorm(x, self.w[self.tensor], self.eps, out, rows)
+        ops.rmsnorm(x, self.weight, self.eps, out, rows)
         return out
 
     def fold(self):
-        return NormFold("rms", self.w[self.tensor], self.eps)
+        return NormFold("rms", self.weight, self.eps)
 
 
 @register_part("norm", "layernorm")

@@ -71,6 +71,9 @@ def _register_builtin():
     from .config.morarax import MoraraxConfig
     from .models.morarax import build_morarax
     register_architecture(MoraraxConfig.architecture, MoraraxConfig, build_morarax)
+    from .config.kodezen import KodezenConfig
+    from .models.kodezen import build_kodezen
+    register_architecture(KodezenConfig.architecture, KodezenConfig, build_kodezen)
 
 
 _register_builtin()
