@@ -19,7 +19,7 @@ part of a step that the host spends planning and launching, which the look-ahead
 another prompt is prefilled 256 tokens a step; with --pressure SHARE, the batch in a pool too small for its
 requests at the headline sizes.
 
-    python bench.py --design megozen|bogilix|morarax [--sizes s,m,l] [--design-batches 1,8,64]
+    python bench.py --design megozen|bogilix|morarax|kodezen [--sizes s,m,l] [--design-batches 1,8,64]
 
 times the Megozen presets instead (latent attention, routed experts), each beside the dense model of equal width,
 layers, vocabulary and work per token, and prints a line of its own; the default workload above is untouched.
@@ -283,7 +283,8 @@ def second_model_points(preset, dtype, element, batch, context, prefill_tokens, 
 def design_points(design: str, sizes: list[str], dtype: str, dtype_name: str, batches: list[int], context: int,
                   prefill_tokens: int, steps: int, warmup: int, which: str = "both") -> dict:
     """Decode and prefill throughput of another design's presets (`<design>-<size>`) beside the dense model of equal
-    width, layers, vocabulary and work per token (`<design>-<size>-dense`), random weights, every layer."""
+    width, layers, vocabulary and work per token (`<design>-<size>-dense`; where the presets name a `<design>-<size>-twin`
+    instead, the closest other design at equal size), random weights, every layer."""
     import gc
     import torch
     from sprout_lm_amd.cli import PRESETS
@@ -291,7 +292,8 @@ def design_points(design: str, sizes: list[str], dtype: str, dtype_name: str, ba
     element = 2 if dtype_name == "bf16" else 4
     out = {}
     for size in sizes:
-        for name in ([f"{design}-{size}"] if which != "dense" else []) + ([f"{design}-{size}-dense"] if which != "design" else []):
+        twin = f"{design}-{size}-dense" if f"{design}-{size}-dense" in PRESETS else f"{design}-{size}-twin"
+        for name in ([f"{design}-{size}"] if which != "dense" else []) + ([twin] if which != "design" else []):
             gc.collect()
             torch.cuda.empty_cache()
             cfg = config_from_dict(dict(PRESETS[name]))
@@ -314,7 +316,7 @@ def design_points(design: str, sizes: list[str], dtype: str, dtype_name: str, ba
 
 def main() -> int:
     parser = argparse.ArgumentParser()
-    parser.add_argument("--design", default=None, choices=["megozen", "bogilix", "morarax"],
+    parser.add_argument("--design", default=None, choices=["megozen", "bogilix", "morarax", "kodezen"],
                         help="time nothing but this design's presets (--sizes) beside dense models of equal size: "
                              "decode at --design-batches and --context, prefill of --prefill-tokens; prints a line of its own")
     parser.add_argument("--sizes", default="s,m,l", help="with --design: which of its presets")

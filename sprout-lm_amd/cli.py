@@ -2,7 +2,7 @@
 
     python -m sprout_lm_amd demo [--json] [--pressure]
     python -m sprout_lm_amd generate MODEL_DIR --prompt-ids 1,2,3 [--max-new-tokens N] ...
-    python -m sprout_lm_amd init --preset tiny-a|tiny-b|qwen2.5-0.5b|megozen-s|bogilix-s|morarax-s|... | --config FILE  --out DIR [--seed N]
+    python -m sprout_lm_amd init --preset tiny-a|tiny-b|qwen2.5-0.5b|megozen-s|bogilix-s|morarax-s|kodezen-s|... | --config FILE  --out DIR [--seed N]
 
 `demo` is the counterpart of the reference's src/demo.ts, with the reference's two options: a few requests on a
 tiny random model, told round by round (--json: the same as one JSON document; --pressure: a pool so small that
@@ -141,6 +141,35 @@ PRESETS.update({
     # large: 8 layers of width 4,096; attention of 32 heads of 128 over 4 key/value heads, retention of 32 heads
     "morarax-l": _morarax_preset(4096, 8, 32, 4, 128, 32, 16, 8192, 32768),
     "morarax-l-dense": _dense_twin(4096, 8, 32, 4, 8192, 32768),
+})
+
+
+def _kodezen_preset(width: int, layers: int, heads: int, kv_heads: int, dim: int, ff: int, vocab: int) -> dict:
+    """A Kodezen configuration: layers in the order mamba2, attention, mamba2, mamba1, again and again.  The state-space
+    mixers are twice as wide as the model (mamba2: heads of 64 values, a state of 128 rows, two groups; mamba1: a state of
+    16); attention heads of `dim` of which half turn, a window of 1,024 keys that keeps the first four.  Feed-forwards take
+    turns: dense with `ff` * 3 / 2 inner numbers (two matrices where a gated one has three), and two of eight experts of
+    `ff` / 2."""
+    mamba2 = {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 2, "conv": 4, "norm_groups": 2}
+    mamba1 = {"inner": 2 * width, "state": 16, "dt_rank": width // 16, "conv": 4}
+    attention = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "conv": 3,
+                 "rot": {"base": 500000.0, "dims": dim // 2}, "mask": {"size": 1024, "keep_first": 4}}
+    order = (("mamba2", mamba2), ("attention", attention), ("mamba2", mamba2), ("mamba1", mamba1))
+    dense = {"kind": "dense", "ff": ff * 3 // 2}
+    moe = {"kind": "moe", "expert": {"ff": ff // 2}, "router": {"experts": 8, "top": 2}}
+    entries = [{"type": order[i % 4][0], "mixer": order[i % 4][1], "mlp": moe if i % 2 else dense} for i in range(layers)]
+    return {"architecture": "Kodezen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "embedding": {"scale": width ** 0.5},
+            "canon": {"taps": 4}, "layers": entries}
+
+
+PRESETS.update({
+    # beside each the closest design the engine has at equal width, layers, attention heads and feed-forward work: Morarax
+    "kodezen-s": _kodezen_preset(1024, 8, 16, 2, 64, 2048, 32768),
+    "kodezen-s-twin": _morarax_preset(1024, 8, 16, 2, 64, 8, 16, 2048, 32768),
+    "kodezen-m": _kodezen_preset(2048, 12, 16, 2, 128, 4224, 32768),
+    "kodezen-m-twin": _morarax_preset(2048, 12, 16, 2, 128, 16, 16, 4224, 32768),
+    "kodezen-l": _kodezen_preset(4096, 8, 32, 4, 128, 8192, 32768),
+    "kodezen-l-twin": _morarax_preset(4096, 8, 32, 4, 128, 32, 16, 8192, 32768),
 })
 
 

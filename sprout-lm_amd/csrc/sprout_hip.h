@@ -322,7 +322,10 @@ int sp_scale_rows(void* stream, int dtype, const void* x, const float* weights, 
 int sp_ssd_scan(void* stream, int dtype, const void* proj, long long proj_stride, int z_off, int dt_off, const void* xbc,
                 long long xbc_stride, int heads, int vdim, int state_size, int groups, const float* dt_bias, const float* a_log,
                 const float* skip, const int32_t* q_start, const int32_t* q_len, const int32_t* state_slots, float* state,
-                float* out, int T, int n_seqs);
+                float* out, int T, int n_seqs, int max_q_len, float* scratch);
+// max_q_len: the most tokens one request brings to the step; scratch: float32 scratch of sp_ssd_scan_scratch_floats numbers
+// (null, or a short longest portion: every request's tokens are walked in one go, else in chunks side by side).
+long long sp_ssd_scan_scratch_floats(int heads, int vdim, int state_size, int n_seqs, int max_q_len);
 // Selective scan (Mamba).  Per channel c and token t: d = softplus(dt[t, c]) (dt float32 [T, inner], bias included),
 //   S[c, :] <- exp(d a[c, :]) S[c, :] + d u[t, c] B_t,  y = S[c, :] . C_t + skip[c] u[t, c],  out[t, c] = y * silu(z[t, c]).
 // u [T, u_stride] from u_off, z likewise, B and C (state numbers each) the columns of bc [T, bc_stride] from bc_off on, all
@@ -331,7 +334,9 @@ int sp_ssd_scan(void* stream, int dtype, const void* proj, long long proj_stride
 int sp_selective_scan(void* stream, int dtype, const void* u, long long u_stride, int u_off, const void* z, long long z_stride,
                       int z_off, const float* dt, const void* bc, long long bc_stride, int bc_off, int inner, int state_size,
                       const float* a, const float* skip, const int32_t* q_start, const int32_t* q_len,
-                      const int32_t* state_slots, float* state, void* out, int T, int n_seqs);
+                      const int32_t* state_slots, float* state, void* out, int T, int n_seqs, int max_q_len, float* scratch);
+// max_q_len, scratch: as for sp_ssd_scan, with sp_selective_scan_scratch_floats numbers.
+long long sp_selective_scan_scratch_floats(int inner, int state_size, int n_seqs, int max_q_len);
 // Queries and keys of attention whose heads' weights are mixed after the softmax.  qk [T, (nq + nkv) * dim] of `dtype`
 // holds q then k.  Every head is divided by its root mean square (eps inside the root) and multiplied by q_norm or k_norm
 // (dim numbers of w_dtype), then the first rotary_dim numbers turn, 2i with 2i + 1, by positions[t] * freq[i] (float64

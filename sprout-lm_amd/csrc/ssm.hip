@@ -118,62 +118,109 @@ struct SsdArgs {
   const int32_t* state_slots;
   float* state;
   float* out;
+  int chunk, chunks;           // tokens a chunk, chunks a request (the longest portion's), where portions are walked in chunks
+  float* scratch;              // [requests * chunks, heads, state, vdim]
+  float* step_sums;            // [requests * chunks, heads]
 };
 
 // A block per request and 32 columns of the heads' values; a column's state rows are shared out over 8 neighbouring lanes
 // (lane rg holds rows rg, rg + 8, ...: KPT of them), so a token's output is a sum over those lanes alone and the walk along
 // the request's tokens needs no barrier.  Columns are independent of each other: S[:, p] takes B and u_p only.
-template <typename T, int KPT>
+//
+// Long portions are walked in chunks of `chunk` tokens side by side, in three passes over the same recurrence:
+//   MODE 1  every chunk from a state of zeros: what it adds, U_c, and the sum of its step sizes (the chunk's decay is
+//           exp(-rate * sum)) go to the scratch;
+//   carry   per state element the chunks in turn, S <- decay_c S + U_c, leaving in U_c's place the state chunk c starts
+//           from, and in the request's state rows the state after its last token;
+//   MODE 2  every chunk again, from the state it starts from, with the outputs.
+// MODE 0 walks a request's tokens in one go (short portions, single tokens).  blockIdx.y: the request (MODE 0), or
+// request * chunks_per_request + chunk.
+template <typename T, int KPT, int MODE>
 __global__ __launch_bounds__(256) void ssd_scan_kernel(SsdArgs a) {
-  const int s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rg = lane & 7, pc = lane >> 3;
   const int inner = a.heads * a.vdim, N = a.state_size;
+  const int s = MODE == 0 ? blockIdx.y : blockIdx.y / a.chunks;
+  const int ci = MODE == 0 ? 0 : blockIdx.y % a.chunks;
   int col = blockIdx.x * 32 + wave * 8 + pc;
   const bool live = col < inner;
   if (!live) col = inner - 1;      // the lane stays for its neighbours' sums and stores nothing
   const int n = col / a.vdim, p = col % a.vdim, g = n / (a.heads / a.groups);
-  const int q0 = a.q_start[s], L = a.q_len[s];
+  int q0 = a.q_start[s], L = a.q_len[s];
+  if (MODE != 0) {
+    q0 += ci * a.chunk;
+    L = min(a.chunk, L - ci * a.chunk);
+  }
   if (L <= 0) return;
-  float* S = a.state + ((size_t(a.state_slots[s]) * a.heads + n) * N) * a.vdim + p;
+  // the state rows of this column: the request's own (MODE 0), or the chunk's place in the scratch
+  float* S = MODE == 0 ? a.state + ((size_t(a.state_slots[s]) * a.heads + n) * N) * a.vdim + p
+                       : a.scratch + ((size_t(blockIdx.y) * a.heads + n) * N) * a.vdim + p;
   float st[KPT];
 #pragma unroll
   for (int k = 0; k < KPT; ++k) {
     const int r = rg + 8 * k;
-    st[k] = r < N ? S[size_t(r) * a.vdim] : 0.f;
+    st[k] = (MODE != 1 && r < N) ? S[size_t(r) * a.vdim] : 0.f;
   }
   const float rate = expf(a.a_log[n]), bias = a.dt_bias[n], skip = a.skip[n];
   const T* proj = (const T*)a.proj;
   const T* xbc = (const T*)a.xbc;
   const int b_off = inner + g * N, c_off = inner + a.groups * N + g * N;
+  float steps = 0.f;
   for (int t = q0; t < q0 + L; ++t) {
     const T* pr = proj + size_t(t) * a.proj_stride;
     const T* xr = xbc + size_t(t) * a.xbc_stride;
     const float d = softplus_of(to_float(pr[a.dt_off + n]) + bias);
     const float decay = expf(-rate * d);
     const float u = to_float(xr[col]);
-    const float z = to_float(pr[a.z_off + col]);
     const float du = d * u;
+    steps += d;
     float y = 0.f;
 #pragma unroll
     for (int k = 0; k < KPT; ++k) {
       const int r = rg + 8 * k;
       if (r < N) {
         st[k] = fmaf(decay, st[k], du * to_float(xr[b_off + r]));
-        y = fmaf(st[k], to_float(xr[c_off + r]), y);
+        if (MODE != 1) y = fmaf(st[k], to_float(xr[c_off + r]), y);
       }
     }
-    y += __shfl_xor(y, 1, 64);
-    y += __shfl_xor(y, 2, 64);
-    y += __shfl_xor(y, 4, 64);
-    if (rg == 0 && live) a.out[size_t(t) * inner + col] = fmaf(skip, u, y) * silu_of(z);
+    if (MODE != 1) {
+      y += __shfl_xor(y, 1, 64);
+      y += __shfl_xor(y, 2, 64);
+      y += __shfl_xor(y, 4, 64);
+      if (rg == 0 && live) a.out[size_t(t) * inner + col] = fmaf(skip, u, y) * silu_of(to_float(pr[a.z_off + col]));
+    }
   }
+  if (MODE == 2) return;
   if (live) {
 #pragma unroll
     for (int k = 0; k < KPT; ++k) {
       const int r = rg + 8 * k;
       if (r < N) S[size_t(r) * a.vdim] = st[k];
     }
+    if (MODE == 1 && p == 0 && rg == 0) a.step_sums[size_t(blockIdx.y) * a.heads + n] = steps;
   }
+}
+
+// A thread a state element of a request: the chunks in turn.
+__global__ __launch_bounds__(256) void ssd_carry_kernel(SsdArgs a) {
+  const int s = blockIdx.y;
+  const size_t per_head = size_t(a.state_size) * a.vdim, per_request = per_head * a.heads;
+  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= per_request) return;
+  const int L = a.q_len[s];
+  if (L <= 0) return;
+  const int n = int(e / per_head), used = (L + a.chunk - 1) / a.chunk;
+  const float rate = expf(a.a_log[n]);
+  float* mine = a.state + size_t(a.state_slots[s]) * per_request + e;
+  float S = *mine;
+  for (int c = 0; c < used; ++c) {
+    const size_t number = size_t(s) * a.chunks + c;
+    float* at = a.scratch + number * per_request + e;
+    const float added = *at;
+    *at = S;
+    S = fmaf(expf(-rate * a.step_sums[number * a.heads + n]), S, added);
+  }
+  *mine = S;
 }
 
 // ------------------------------------------------------------------------------------------------ selective scan
@@ -195,58 +242,96 @@ struct SelArgs {
   const int32_t* state_slots;
   float* state;
   void* out;
+  int chunk, chunks;
+  float* scratch;              // [requests * chunks, inner, state]
+  float* step_sums;            // [requests * chunks, inner]
 };
 
 // A block per request and 64 channels; a channel's states are shared out over 4 neighbouring lanes (lane ng holds states ng,
-// ng + 4, ...: KPT of them).
-template <typename T, int KPT>
+// ng + 4, ...: KPT of them).  MODE as for the duality scan: long portions in chunks side by side, three passes; a chunk's
+// decay of state (c, n) is exp(rate[c, n] * the sum of the channel's step sizes).
+template <typename T, int KPT, int MODE>
 __global__ __launch_bounds__(256) void selective_scan_kernel(SelArgs a) {
-  const int s = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int ng = lane & 3, cc = lane >> 2;
   const int N = a.state_size;
+  const int s = MODE == 0 ? blockIdx.y : blockIdx.y / a.chunks;
+  const int ci = MODE == 0 ? 0 : blockIdx.y % a.chunks;
   int c = blockIdx.x * 64 + wave * 16 + cc;
   const bool live = c < a.inner;
   if (!live) c = a.inner - 1;
-  const int q0 = a.q_start[s], L = a.q_len[s];
+  int q0 = a.q_start[s], L = a.q_len[s];
+  if (MODE != 0) {
+    q0 += ci * a.chunk;
+    L = min(a.chunk, L - ci * a.chunk);
+  }
   if (L <= 0) return;
-  float* S = a.state + (size_t(a.state_slots[s]) * a.inner + c) * N;
+  float* S = MODE == 0 ? a.state + (size_t(a.state_slots[s]) * a.inner + c) * N
+                       : a.scratch + (size_t(blockIdx.y) * a.inner + c) * N;
   float st[KPT], ak[KPT];
 #pragma unroll
   for (int k = 0; k < KPT; ++k) {
     const int n = ng + 4 * k;
-    st[k] = n < N ? S[n] : 0.f;
+    st[k] = (MODE != 1 && n < N) ? S[n] : 0.f;
     ak[k] = n < N ? a.a[size_t(c) * N + n] : 0.f;
   }
   const float skip = a.skip[c];
   const T* up = (const T*)a.u + a.u_off + c;
   const T* zp = (const T*)a.z + a.z_off + c;
   const T* bc = (const T*)a.bc + a.bc_off;
+  float steps = 0.f;
   for (int t = q0; t < q0 + L; ++t) {
     const float d = softplus_of(a.dt[size_t(t) * a.inner + c]);
     const float u = to_float(up[size_t(t) * a.u_stride]);
-    const float z = to_float(zp[size_t(t) * a.z_stride]);
     const T* row = bc + size_t(t) * a.bc_stride;
     const float du = d * u;
+    steps += d;
     float y = 0.f;
 #pragma unroll
     for (int k = 0; k < KPT; ++k) {
       const int n = ng + 4 * k;
       if (n < N) {
         st[k] = fmaf(expf(d * ak[k]), st[k], du * to_float(row[n]));
-        y = fmaf(st[k], to_float(row[N + n]), y);
+        if (MODE != 1) y = fmaf(st[k], to_float(row[N + n]), y);
       }
     }
-    y += __shfl_xor(y, 1, 64);
-    y += __shfl_xor(y, 2, 64);
-    if (ng == 0 && live) ((T*)a.out)[size_t(t) * a.inner + c] = from_float<T>(fmaf(skip, u, y) * silu_of(z));
+    if (MODE != 1) {
+      y += __shfl_xor(y, 1, 64);
+      y += __shfl_xor(y, 2, 64);
+      if (ng == 0 && live)
+        ((T*)a.out)[size_t(t) * a.inner + c] = from_float<T>(fmaf(skip, u, y) * silu_of(to_float(zp[size_t(t) * a.z_stride])));
+    }
   }
+  if (MODE == 2) return;
   if (live) {
 #pragma unroll
     for (int k = 0; k < KPT; ++k) {
       const int n = ng + 4 * k;
       if (n < N) S[n] = st[k];
     }
+    if (MODE == 1 && ng == 0) a.step_sums[size_t(blockIdx.y) * a.inner + c] = steps;
   }
+}
+
+__global__ __launch_bounds__(256) void selective_carry_kernel(SelArgs a) {
+  const int s = blockIdx.y;
+  const size_t per_request = size_t(a.inner) * a.state_size;
+  const size_t e = size_t(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= per_request) return;
+  const int L = a.q_len[s];
+  if (L <= 0) return;
+  const int c = int(e / a.state_size), used = (L + a.chunk - 1) / a.chunk;
+  const float rate = a.a[e];
+  float* mine = a.state + size_t(a.state_slots[s]) * per_request + e;
+  float S = *mine;
+  for (int k = 0; k < used; ++k) {
+    const size_t number = size_t(s) * a.chunks + k;
+    float* at = a.scratch + number * per_request + e;
+    const float added = *at;
+    *at = S;
+    S = fmaf(expf(rate * a.step_sums[number * a.inner + c]), S, added);
+  }
+  *mine = S;
 }
 
 // ------------------------------------------------------------------------------------------------ attention with mixed heads
@@ -401,10 +486,28 @@ extern "C" int sp_scale_rows(void* stream, int dtype, const void* x, const float
   return check_launch("sp_scale_rows");
 }
 
+// Portions of more than kScanLong tokens are walked in chunks of kScanChunk.
+constexpr int kScanChunk = 64, kScanLong = 128;
+
+extern "C" long long sp_ssd_scan_scratch_floats(int heads, int vdim, int state_size, int n_seqs, int max_q_len) {
+  if (max_q_len <= kScanLong || n_seqs <= 0) return 0;
+  const long long chunks = (max_q_len + kScanChunk - 1) / kScanChunk;
+  if (n_seqs * chunks > 65535) return 0;      // more chunk numbers than a grid's second dimension counts
+  return (long long)n_seqs * chunks * heads * ((long long)state_size * vdim + 1);
+}
+
+extern "C" long long sp_selective_scan_scratch_floats(int inner, int state_size, int n_seqs, int max_q_len) {
+  if (max_q_len <= kScanLong || n_seqs <= 0) return 0;
+  const long long chunks = (max_q_len + kScanChunk - 1) / kScanChunk;
+  if (n_seqs * chunks > 65535) return 0;
+  return (long long)n_seqs * chunks * inner * ((long long)state_size + 1);
+}
+
 extern "C" int sp_ssd_scan(void* stream, int dtype, const void* proj, long long proj_stride, int z_off, int dt_off,
                            const void* xbc, long long xbc_stride, int heads, int vdim, int state_size, int groups,
                            const float* dt_bias, const float* a_log, const float* skip, const int32_t* q_start,
-                           const int32_t* q_len, const int32_t* state_slots, float* state, float* out, int T, int n_seqs) {
+                           const int32_t* q_len, const int32_t* state_slots, float* state, float* out, int T, int n_seqs,
+                           int max_q_len, float* scratch) {
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_ssd_scan: unsupported dtype %d", dtype);
   SP_REQUIRE(heads > 0 && vdim > 0 && groups > 0 && heads % groups == 0 && state_size > 0 && state_size <= 256,
              "sp_ssd_scan: %d heads of %d in %d groups with a state of %d (up to 256)", heads, vdim, groups, state_size);
@@ -414,27 +517,47 @@ extern "C" int sp_ssd_scan(void* stream, int dtype, const void* proj, long long 
   SP_REQUIRE(proj && xbc && dt_bias && a_log && skip && q_start && q_len && state_slots && state && out && T >= 0 && n_seqs >= 0,
              "sp_ssd_scan: null operand");
   if (T == 0 || n_seqs == 0) return 0;
-  const SsdArgs a = {proj, proj_stride, z_off, dt_off, xbc, xbc_stride, heads, vdim, state_size, groups, dt_bias, a_log, skip,
-                     q_start, q_len, state_slots, state, out};
-  const dim3 grid((inner + 31) / 32, n_seqs);
+  SsdArgs a = {proj, proj_stride, z_off, dt_off, xbc, xbc_stride, heads, vdim, state_size, groups, dt_bias, a_log, skip,
+               q_start, q_len, state_slots, state, out, 0, 1, nullptr, nullptr};
   hipStream_t s = (hipStream_t)stream;
-#define SP_SSD(KPT)                                                         \
-  do {                                                                      \
-    if (dtype == kF32) ssd_scan_kernel<float, KPT><<<grid, 256, 0, s>>>(a); \
-    else ssd_scan_kernel<bf16_t, KPT><<<grid, 256, 0, s>>>(a);              \
+#define SP_SSD_MODE(KPT, MODE)                                                       \
+  do {                                                                               \
+    if (dtype == kF32) ssd_scan_kernel<float, KPT, MODE><<<grid, 256, 0, s>>>(a);    \
+    else ssd_scan_kernel<bf16_t, KPT, MODE><<<grid, 256, 0, s>>>(a);                 \
   } while (0)
-  if (state_size <= 32) SP_SSD(4);
-  else if (state_size <= 64) SP_SSD(8);
-  else if (state_size <= 128) SP_SSD(16);
-  else SP_SSD(32);
+#define SP_SSD(MODE)                                  \
+  do {                                                \
+    if (state_size <= 32) SP_SSD_MODE(4, MODE);       \
+    else if (state_size <= 64) SP_SSD_MODE(8, MODE);  \
+    else if (state_size <= 128) SP_SSD_MODE(16, MODE);\
+    else SP_SSD_MODE(32, MODE);                       \
+  } while (0)
+  const long long need = sp_ssd_scan_scratch_floats(heads, vdim, state_size, n_seqs, max_q_len);
+  if (need == 0 || !scratch) {
+    const dim3 grid((inner + 31) / 32, n_seqs);
+    SP_SSD(0);
+    return check_launch("sp_ssd_scan");
+  }
+  a.chunk = kScanChunk;
+  a.chunks = (max_q_len + kScanChunk - 1) / kScanChunk;
+  a.scratch = scratch;
+  a.step_sums = scratch + size_t(n_seqs) * a.chunks * heads * state_size * vdim;
+  const dim3 grid((inner + 31) / 32, n_seqs * a.chunks);
+  SP_SSD(1);
+  if (check_launch("sp_ssd_scan (chunks)")) return 1;
+  ssd_carry_kernel<<<dim3((size_t(inner) * state_size + 255) / 256, n_seqs), 256, 0, s>>>(a);
+  if (check_launch("sp_ssd_scan (carry)")) return 1;
+  SP_SSD(2);
 #undef SP_SSD
-  return check_launch("sp_ssd_scan");
+#undef SP_SSD_MODE
+  return check_launch("sp_ssd_scan (outputs)");
 }
 
 extern "C" int sp_selective_scan(void* stream, int dtype, const void* u, long long u_stride, int u_off, const void* z,
                                  long long z_stride, int z_off, const float* dt, const void* bc, long long bc_stride, int bc_off,
                                  int inner, int state_size, const float* a, const float* skip, const int32_t* q_start,
-                                 const int32_t* q_len, const int32_t* state_slots, float* state, void* out, int T, int n_seqs) {
+                                 const int32_t* q_len, const int32_t* state_slots, float* state, void* out, int T, int n_seqs,
+                                 int max_q_len, float* scratch) {
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_selective_scan: unsupported dtype %d", dtype);
   SP_REQUIRE(inner > 0 && state_size > 0 && state_size <= 256, "sp_selective_scan: %d channels with a state of %d (up to 256)",
              inner, state_size);
@@ -443,22 +566,41 @@ extern "C" int sp_selective_scan(void* stream, int dtype, const void* u, long lo
   SP_REQUIRE(u && z && dt && bc && a && skip && q_start && q_len && state_slots && state && out && T >= 0 && n_seqs >= 0,
              "sp_selective_scan: null operand");
   if (T == 0 || n_seqs == 0) return 0;
-  const SelArgs args = {u, u_stride, u_off, z, z_stride, z_off, dt, bc, bc_stride, bc_off, inner, state_size, a, skip,
-                        q_start, q_len, state_slots, state, out};
-  const dim3 grid((inner + 63) / 64, n_seqs);
+  SelArgs args = {u, u_stride, u_off, z, z_stride, z_off, dt, bc, bc_stride, bc_off, inner, state_size, a, skip,
+                  q_start, q_len, state_slots, state, out, 0, 1, nullptr, nullptr};
   hipStream_t s = (hipStream_t)stream;
-#define SP_SEL(KPT)                                                                  \
-  do {                                                                               \
-    if (dtype == kF32) selective_scan_kernel<float, KPT><<<grid, 256, 0, s>>>(args); \
-    else selective_scan_kernel<bf16_t, KPT><<<grid, 256, 0, s>>>(args);              \
+#define SP_SEL_MODE(KPT, MODE)                                                             \
+  do {                                                                                     \
+    if (dtype == kF32) selective_scan_kernel<float, KPT, MODE><<<grid, 256, 0, s>>>(args); \
+    else selective_scan_kernel<bf16_t, KPT, MODE><<<grid, 256, 0, s>>>(args);              \
   } while (0)
-  if (state_size <= 16) SP_SEL(4);
-  else if (state_size <= 32) SP_SEL(8);
-  else if (state_size <= 64) SP_SEL(16);
-  else if (state_size <= 128) SP_SEL(32);
-  else SP_SEL(64);
+#define SP_SEL(MODE)                                   \
+  do {                                                 \
+    if (state_size <= 16) SP_SEL_MODE(4, MODE);        \
+    else if (state_size <= 32) SP_SEL_MODE(8, MODE);   \
+    else if (state_size <= 64) SP_SEL_MODE(16, MODE);  \
+    else if (state_size <= 128) SP_SEL_MODE(32, MODE); \
+    else SP_SEL_MODE(64, MODE);                        \
+  } while (0)
+  const long long need = sp_selective_scan_scratch_floats(inner, state_size, n_seqs, max_q_len);
+  if (need == 0 || !scratch) {
+    const dim3 grid((inner + 63) / 64, n_seqs);
+    SP_SEL(0);
+    return check_launch("sp_selective_scan");
+  }
+  args.chunk = kScanChunk;
+  args.chunks = (max_q_len + kScanChunk - 1) / kScanChunk;
+  args.scratch = scratch;
+  args.step_sums = scratch + size_t(n_seqs) * args.chunks * inner * state_size;
+  const dim3 grid((inner + 63) / 64, n_seqs * args.chunks);
+  SP_SEL(1);
+  if (check_launch("sp_selective_scan (chunks)")) return 1;
+  selective_carry_kernel<<<dim3((size_t(inner) * state_size + 255) / 256, n_seqs), 256, 0, s>>>(args);
+  if (check_launch("sp_selective_scan (carry)")) return 1;
+  SP_SEL(2);
 #undef SP_SEL
-  return check_launch("sp_selective_scan");
+#undef SP_SEL_MODE
+  return check_launch("sp_selective_scan (outputs)");
 }
 
 extern "C" int sp_qk_cross_prepare(void* stream, int dtype, const void* qk, int nq, int nkv, int dim, int width, int w_dtype,

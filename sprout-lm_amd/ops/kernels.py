@@ -901,9 +901,22 @@ def scale_rows(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) -> Non
     check(library().sp_scale_rows(_stream(), _code(x, "rows"), x.data_ptr(), weights.data_ptr(), top, out.data_ptr(), T, H))
 
 
+def _scan_scratch(need: int, workspace):
+    """The scratch of a scan that walks long portions in chunks: None where the step needs none or the caller has none."""
+    if not need or workspace is None:
+        return None
+    scratch = workspace(need)
+    if scratch.dtype != torch.float32 or scratch.numel() < need or not scratch.is_cuda:
+        raise KernelError("scan: workspace too small")
+    return scratch
+
+
 def ssd_scan(proj: torch.Tensor, z_off: int, dt_off: int, xbc: torch.Tensor, heads: int, vdim: int, state_size: int, groups: int,
-             dt_bias, a_log, skip, q_start, q_len, state_slots, n_seqs: int, state: torch.Tensor, out: torch.Tensor) -> None:
-    """The state-space-duality scan of sp_ssd_scan (sprout_hip.h); out float32 [T, heads * vdim] = y * silu(z)."""
+             dt_bias, a_log, skip, q_start, q_len, state_slots, n_seqs: int, state: torch.Tensor, out: torch.Tensor,
+             max_q_len: int = 0, workspace=None) -> None:
+    """The state-space-duality scan of sp_ssd_scan (sprout_hip.h); out float32 [T, heads * vdim] = y * silu(z).
+    `max_q_len`: the most tokens one request brings (0: unknown); with `workspace(n)` (a float32 device tensor of at least
+    n elements) long portions are walked in chunks side by side."""
     for t, what in ((proj, "projections"), (xbc, "convolved rows"), (state, "state"), (out, "scan output")):
         _gpu(t, what)
     T, inner = out.shape[0], heads * vdim
@@ -917,16 +930,19 @@ def ssd_scan(proj: torch.Tensor, z_off: int, dt_off: int, xbc: torch.Tensor, hea
     if state.dtype != torch.float32 or tuple(state.shape[1:]) != (heads, state_size, vdim) or not state.is_contiguous():
         raise KernelError(f"ssd_scan: the state must be float32 [slots, {heads}, {state_size}, {vdim}]")
     _step_ints(q_start, q_len, state_slots, n_seqs)
+    scratch = _scan_scratch(library().sp_ssd_scan_scratch_floats(heads, vdim, state_size, n_seqs, int(max_q_len)), workspace)
     check(library().sp_ssd_scan(_stream(), _code(proj, "projections"), proj.data_ptr(), proj.stride(0), z_off, dt_off,
                                 xbc.data_ptr(), xbc.stride(0), heads, vdim, state_size, groups, dt_bias.data_ptr(),
                                 a_log.data_ptr(), skip.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), state_slots.data_ptr(),
-                                state.data_ptr(), out.data_ptr(), T, n_seqs))
+                                state.data_ptr(), out.data_ptr(), T, n_seqs, int(max_q_len) if scratch is not None else 0,
+                                _ptr(scratch)))
 
 
 def selective_scan(u: torch.Tensor, u_off: int, z: torch.Tensor, z_off: int, dt: torch.Tensor, bc: torch.Tensor, bc_off: int,
                    inner: int, state_size: int, a, skip, q_start, q_len, state_slots, n_seqs: int, state: torch.Tensor,
-                   out: torch.Tensor) -> None:
-    """The selective scan of sp_selective_scan (sprout_hip.h); out [T, inner] of the rows' dtype = y * silu(z)."""
+                   out: torch.Tensor, max_q_len: int = 0, workspace=None) -> None:
+    """The selective scan of sp_selective_scan (sprout_hip.h); out [T, inner] of the rows' dtype = y * silu(z).
+    `max_q_len`, `workspace`: as for ssd_scan."""
     for t, what in ((u, "inputs"), (z, "gates"), (dt, "step sizes"), (bc, "B and C"), (state, "state"), (out, "scan output")):
         _gpu(t, what)
     T = out.shape[0]
@@ -940,10 +956,12 @@ def selective_scan(u: torch.Tensor, u_off: int, z: torch.Tensor, z_off: int, dt:
     if state.dtype != torch.float32 or tuple(state.shape[1:]) != (inner, state_size) or not state.is_contiguous():
         raise KernelError(f"selective_scan: the state must be float32 [slots, {inner}, {state_size}]")
     _step_ints(q_start, q_len, state_slots, n_seqs)
+    scratch = _scan_scratch(library().sp_selective_scan_scratch_floats(inner, state_size, n_seqs, int(max_q_len)), workspace)
     check(library().sp_selective_scan(_stream(), _code(u, "inputs"), u.data_ptr(), u.stride(0), u_off, z.data_ptr(), z.stride(0),
                                       z_off, dt.data_ptr(), bc.data_ptr(), bc.stride(0), bc_off, inner, state_size, a.data_ptr(),
                                       skip.data_ptr(), q_start.data_ptr(), q_len.data_ptr(), state_slots.data_ptr(),
-                                      state.data_ptr(), out.data_ptr(), T, n_seqs))
+                                      state.data_ptr(), out.data_ptr(), T, n_seqs, int(max_q_len) if scratch is not None else 0,
+                                      _ptr(scratch)))
 
 
 def qk_cross_prepare(qk: torch.Tensor, nq: int, nkv: int, dim: int, width: int, q_norm, k_norm, eps: float, positions, freq,

@@ -87,9 +87,9 @@ def _declare(lib):
         "sp_activation": [c_void, c_int, c_void, c_i64, c_int],
         "sp_scale_rows": [c_void, c_int, c_void, c_void, c_int, c_void, c_int, c_int],
         "sp_ssd_scan": [c_void, c_int, c_void, c_i64, c_int, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_void, c_void,
-                        c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
+                        c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "sp_selective_scan": [c_void, c_int, c_void, c_i64, c_int, c_void, c_i64, c_int, c_void, c_void, c_i64, c_int, c_int,
-                              c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
+                              c_int, c_void, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "sp_qk_cross_prepare": [c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_int, c_void, c_void, c_float, c_void,
                                 c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int],
         "sp_head_mix": [c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_void, c_int],
@@ -102,6 +102,10 @@ def _declare(lib):
     lib.sp_rglru_carry_floats.restype = c_i64
     lib.sp_retention_scratch_floats.argtypes = [c_int] * 6
     lib.sp_retention_scratch_floats.restype = c_i64
+    lib.sp_ssd_scan_scratch_floats.argtypes = [c_int] * 5
+    lib.sp_ssd_scan_scratch_floats.restype = c_i64
+    lib.sp_selective_scan_scratch_floats.argtypes = [c_int] * 4
+    lib.sp_selective_scan_scratch_floats.restype = c_i64
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
         fn.argtypes = argtypes

@@ -15,7 +15,7 @@ from .sink_attention import padded_width
 
 @register_part("mixer", "mixed_heads_attention")
 class MixedHeadsAttention(Mixer):
-    """q = conv(W_q h), k = conv(W_k h): a causal convolution of `taps` taps per channel, no bias (`taps` 1: none).  The
+    """q = conv(W_q h), k = conv(W_k h): a causal convolution of `taps` taps per channel, no bias (one tap: a factor per channel).  The
     values are the keys as they leave the convolution.  Every q and k head is then RMS-normed over `dim` with a weight of
     that size shared by the heads (`eps` inside the root), and `position` (neighbouring pairs) turns its first numbers.
     score = (q . k) * scale; position i sees j <= i with i - j < window (None: all) or j < keep_first; ordinary softmax.
@@ -54,12 +54,12 @@ class MixedHeadsAttention(Mixer):
         self.page_tokens = page_tokens
         self.names = tuple(tensors)
         self.channels = (heads + kv_heads) * dim
-        self.conv = ShortConv(self.channels, taps, tensor="conv") if taps > 1 else None
+        self.conv = ShortConv(self.channels, taps, tensor="conv")
 
     def cache_spec(self):
         spec = {"pages": PagedKVSpec(self.kv_heads * self.kv_heads, self.width, self.window, self.page_tokens,
                                      keep_first=self.keep_first)}
-        if self.conv is not None:
+        if self.taps > 1:
             spec["inputs"] = self.conv.cache_spec()
         return spec
 
@@ -75,16 +75,14 @@ class MixedHeadsAttention(Mixer):
         H, G, D = self.heads, self.kv_heads, self.dim
         out = {q: TensorSpec((H * D, self.hidden)), k: TensorSpec((G * D, self.hidden)),
                q + norm: TensorSpec((D,), "vector", "one_plus_normal"), k + norm: TensorSpec((D,), "vector", "one_plus_normal"),
-               talk: TensorSpec((H, H), "vector", "one_plus_normal"), o: TensorSpec((self.hidden, H * D))}
-        if self.conv is not None:
-            out.update({q + conv: TensorSpec((H * D, self.taps), "vector"), k + conv: TensorSpec((G * D, self.taps), "vector")})
+               talk: TensorSpec((H, H), "vector", "one_plus_normal"), o: TensorSpec((self.hidden, H * D)),
+               q + conv: TensorSpec((H * D, self.taps), "vector"), k + conv: TensorSpec((G * D, self.taps), "vector")}
         return out
 
     def bind(self, tensors):
         q, k, conv, norm, talk, o = self.names
         self.w_qk = torch.cat([tensors[q], tensors[k]], dim=0).contiguous()
-        if self.conv is not None:
-            self.conv.bind({"conv": torch.cat([tensors[q + conv], tensors[k + conv]], dim=0).contiguous()})
+        self.conv.bind({"conv": torch.cat([tensors[q + conv], tensors[k + conv]], dim=0).contiguous()})
         self.w_q_norm, self.w_k_norm = tensors[q + norm].contiguous(), tensors[k + norm].contiguous()
         self.talk = tensors[talk].to(torch.float32).contiguous()
         self.w_o = tensors[o]
@@ -99,12 +97,10 @@ class MixedHeadsAttention(Mixer):
     def forward(self, ctx, h, residual, cache):
         T, H, G, D, W = h.shape[0], self.heads, self.kv_heads, self.dim, self.width
         pages = cache["pages"]
-        qk = ctx.buffer("qk", (T, self.channels), ctx.act_dtype)
-        ops.gemm(h, self.w_qk, qk)
-        if self.conv is not None:
-            raw = qk
-            qk = ctx.buffer("qk_conv", (T, self.channels), ctx.act_dtype)
-            self.conv.forward(ctx, raw, qk, cache["inputs"])
+        raw = ctx.buffer("qk", (T, self.channels), ctx.act_dtype)
+        ops.gemm(h, self.w_qk, raw)
+        qk = ctx.buffer("qk_conv", (T, self.channels), ctx.act_dtype)
+        self.conv.forward(ctx, raw, qk, cache.get("inputs"))
         queries = ctx.buffer("cross_q", (T, H * G * W), ctx.act_dtype)
         rotary = getattr(self.position, "rotary_dim", 0)
         writes = pages.writes

@@ -77,7 +77,8 @@ class StateSpaceDuality(Mixer):
         self.conv.forward(ctx, proj, xbc, cache.get("inputs"), x_off=inner)
         gated = ctx.buffer("ssd_gated", (T, inner), torch.float32)
         ops.ssd_scan(proj, 0, inner + self.channels, xbc, self.heads, self.vdim, self.state, self.groups, self.dt_bias,
-                     self.a_log, self.skip, ctx.q_start, ctx.q_len, ctx.state_slots, ctx.n_seqs, cache["state"].state, gated)
+                     self.a_log, self.skip, ctx.q_start, ctx.q_len, ctx.state_slots, ctx.n_seqs, cache["state"].state, gated,
+                     max_q_len=ctx.max_q_len, workspace=lambda n: ctx.buffer("scan_chunks", (n,), torch.float32))
         normed = ctx.buffer("ssd_normed", (T, inner), ctx.act_dtype)
         ops.group_rmsnorm(gated, self.w_norm, self.eps, normed, self.norm_groups)
         ops.gemm(normed, self.w_o, residual, accumulate=True)
@@ -151,5 +152,6 @@ class SelectiveScan(Mixer):
         ops.gemm(low, self.w_dt, dt, bias=self.b_dt)
         out = ctx.buffer("scan_out", (T, inner), ctx.act_dtype)
         ops.selective_scan(u, 0, proj, inner, dt, bc, 0, inner, N, self.rates, self.skip, ctx.q_start, ctx.q_len,
-                           ctx.state_slots, ctx.n_seqs, cache["state"].state, out)
+                           ctx.state_slots, ctx.n_seqs, cache["state"].state, out, max_q_len=ctx.max_q_len,
+                           workspace=lambda n: ctx.buffer("scan_chunks", (n,), torch.float32))
         ops.gemm(out, self.w_o, residual, accumulate=True)

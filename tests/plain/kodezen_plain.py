@@ -151,7 +151,7 @@ def attention_mixer(w, pre: str, m, h, positions, eps, store=f32):
     kn = store(rms(k, eps) * np.asarray(w[pre + "k.norm"], dtype=np.float64))
     qn = store(turn_pairs(qn, positions, m["rot"]["dims"], m["rot"]["base"]))
     kn = store(turn_pairs(kn, positions, m["rot"]["dims"], m["rot"]["base"]))
-    mask = visible(T, m["mask"]["size"], m["mask"]["keep_first"])
+    mask = visible(T, m["mask"]["size"], m["mask"]["keep_first"]) if m.get("mask") else visible(T, T + 1, 0)
     weights = np.zeros((H, T, T))
     for n in range(H):
         s = (qn[:, n] @ kn[:, n // (H // G)].T) * float(m["scale"])
