@@ -77,8 +77,8 @@ extern "C" int sp_attention(void* stream, int dtype, const void* q, int q_stride
                             int scores, float softcap, const float* sinks, int mask_chunk, int keep_first) {
   SP_REQUIRE(scores == 0 || (scores == 1 && softcap > 0.f), "sp_attention: no kernel for score stage %d (0 = the scaled product alone, 1 = capped by a positive number)", scores);
   SP_REQUIRE(mask_chunk >= 0, "sp_attention: blocks of %d positions", mask_chunk);
-  SP_REQUIRE(keep_first >= 0 && (keep_first == 0 || kernel_kind == 2),
-             "sp_attention: %d kept first keys need kernel kind 2, the one kernel that knows them", keep_first);
+  SP_REQUIRE(keep_first >= 0 && (keep_first == 0 || kernel_kind == 2 || (kernel_kind == 0 && dtype == kBF16)),
+             "sp_attention: %d kept first keys need the bfloat16 kernels or kernel kind 2, the kernels that know them", keep_first);
   const ScoreStage st = {window, mask_chunk, scores == 1 ? softcap : 0.f, sinks, keep_first};
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_attention: unsupported dtype %d", dtype);
   SP_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "sp_attention: %d query heads do not divide into %d groups", nq, nkv);

@@ -355,7 +355,8 @@ int attention_generic(hipStream_t s, int dtype, const void* q, int q_stride, con
                       const int32_t* q_len, const int32_t* ctx_len, const int32_t* tiles, int n_tiles, void* out,
                       int nq, int nkv, int hd, int page_size, int num_pages, ScoreStage st, float scale, int max_tile_ctx,
                       float* workspace, bool single, bool plain) {
-  SP_REQUIRE(plain || st.keep == 0, "sp_attention: kept first keys are known to the float32-arithmetic kernel alone");
+  SP_REQUIRE(st.keep == 0 || !attention_generic_on_matrix_cores(dtype, nq, nkv, hd, page_size, plain),
+             "sp_attention: the float32 matrix-core kernels do not know kept first keys");
   SP_REQUIRE(int64_t(max_blocks) * page_size < (int64_t(1) << 24),
              "sp_attention: block tables of %d pages of %d tokens exceed the 2^24 positions this kernel counts",
              max_blocks, page_size);

@@ -87,6 +87,19 @@ __device__ __forceinline__ void load_step(KVStep<DT>& r, const PagedKV& kv, int 
   }
 }
 
+// The keys that the step at key0 may be loaded from, for rows that see keys k_lo .. k_hi and the sequence's first `keep`:
+// a step that holds kept first keys is loaded from its own first key on (what lies between the kept keys and k_lo is
+// masked when the step is used; its pages may have been given back, and a page number that is none is clamped), and up
+// to the last kept key only where the step lies wholly before k_lo.
+__device__ __forceinline__ void step_bounds(int key0, int k_lo, int k_hi, int keep, int& lo, int& hi) {
+  lo = k_lo;
+  hi = k_hi;
+  if (keep > key0) {
+    lo = min(k_lo, key0);
+    if (key0 + 32 <= k_lo) hi = min(keep - 1, k_hi);
+  }
+}
+
 constexpr float kNoKeyYet = -1.0e30f;   // running maximum before any key: finite, so that no inf - inf arises
 // The running maximum of a row follows the true maximum only when that has grown by more than this (in
 // log2 units): until then the probabilities are taken against the older maximum and are at most 2^8, which
@@ -120,6 +133,7 @@ __device__ __forceinline__ float max_over_quarters(float x) {
 struct StepRule {
   bool rows_differ;
   float cap_arg, cap_mul;
+  int keep;      // > 0: a sequence's first `keep` keys are visible to every later row, beside the row's own range
 };
 __device__ __forceinline__ StepRule step_rule(const ScoreStage& st, float scale2) {
   StepRule rule;
@@ -127,6 +141,7 @@ __device__ __forceinline__ StepRule step_rule(const ScoreStage& st, float scale2
   const float scale = scale2 / kLog2e;
   rule.cap_arg = st.cap > 0.f ? scale / st.cap : 0.f;
   rule.cap_mul = st.cap > 0.f ? st.cap / scale : 0.f;
+  rule.keep = st.keep;
   return rule;
 }
 // tanh(x) = 1 - 2 / (exp(2x) + 1): exact to a few units of the last place of 1, which a capped score of the
@@ -174,11 +189,25 @@ __device__ __forceinline__ void attend_step_impl(const KVStep<DT>& r, const bf16
       const unsigned limit = span >= 0 ? unsigned(span) : 0u;
       const int base = span >= 0 ? lo : key0 + 64;          // key - base < 0 for every key of the step: none passes
       const int first = key0 + (CONTIG ? 8 : 4) * lj - base;
+      if (rule.keep > 0 && key0 < rule.keep) {      // the same in every lane: a step that holds kept first keys
+        // a second range, 0 .. min(keep - 1, the row's own position), beside the row's own
+        const int hi2 = min(rule.keep - 1, hi);
+        const unsigned limit2 = hi2 >= 0 ? unsigned(hi2) : 0u;
+        const int first2 = key0 + (CONTIG ? 8 : 4) * lj - (hi2 >= 0 ? 0 : key0 + 64);
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+        for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4)
-          s[qt][kt][r4] = unsigned(first + (CONTIG ? 4 : 16) * kt + r4) <= limit ? s[qt][kt][r4] : -INFINITY;
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const int at = (CONTIG ? 4 : 16) * kt + r4;
+            s[qt][kt][r4] = (unsigned(first + at) <= limit || unsigned(first2 + at) <= limit2) ? s[qt][kt][r4] : -INFINITY;
+          }
+      } else {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4)
+            s[qt][kt][r4] = unsigned(first + (CONTIG ? 4 : 16) * kt + r4) <= limit ? s[qt][kt][r4] : -INFINITY;
+      }
     }
     raw[qt] = vmax3(s[qt][0][0], s[qt][0][1], s[qt][0][2]);
     raw[qt] = vmax3(raw[qt], s[qt][0][3], s[qt][1][0]);
@@ -299,11 +328,22 @@ __global__ __launch_bounds__(64) void attention_prefill_kernel(
   const StepRule rule = step_rule(st, scale2);
   // the next step's keys and values are on their way while the current step is multiplied
   KVStep<DT> cur, nxt;
-  int key0 = (k_lo >> 5) << 5;
-  load_step<DT>(cur, kv, key0, k_lo, k_hi);
-  for (; key0 <= k_hi; key0 += 32) {
-    const bool more = key0 + 32 <= k_hi;
-    if (more) load_step<DT>(nxt, kv, key0 + 32, k_lo, k_hi);
+  // the walk: the steps that hold kept first keys, then from the step of the first key the tile's rows see on; the steps
+  // between are skipped
+  const int lo_step = (k_lo >> 5) << 5;
+  const int keep_end = st.keep > 0 ? min(((st.keep + 31) >> 5) << 5, lo_step) : lo_step;
+  auto after = [&](int key) { return key + 32 >= keep_end && key + 32 < lo_step ? lo_step : key + 32; };
+  int key0 = keep_end > 0 && st.keep > 0 ? 0 : lo_step;
+  int lo, hi;
+  step_bounds(key0, k_lo, k_hi, st.keep, lo, hi);
+  load_step<DT>(cur, kv, key0, lo, hi);
+  for (; key0 <= k_hi; key0 = after(key0)) {
+    const int next = after(key0);
+    const bool more = next <= k_hi;
+    if (more) {
+      step_bounds(next, k_lo, k_hi, st.keep, lo, hi);
+      load_step<DT>(nxt, kv, next, lo, hi);
+    }
     attend_step<DT, NQT>(cur, qop, o, m, lsum, key0, k_lo, qpos, qlo, rule, scale2, pos0);
     if (more) cur = nxt;
   }
@@ -673,7 +713,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   const int ctx = ctx_len[seq], pos = ctx - 1;
   const int k_lo = first_visible(pos, st.window, st.chunk);
   const int G = nq / nkv;
-  if (chunk0 > pos || chunk0 + kDecodeChunk <= k_lo) {
+  if (chunk0 > pos || (chunk0 + kDecodeChunk <= k_lo && chunk0 >= st.keep)) {
     // no visible key in this chunk: the merge kernel reads every chunk's (maximum, sum) without looking at
     // the context length, so an empty chunk says so itself
     if (n_splits > 1 && threadIdx.x < G) {
@@ -719,8 +759,10 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
 #pragma unroll
   for (int i = 0; i < kDecodeWaveKeys / 32; ++i) {
     const int key0 = w0 + 32 * i;
-    live[i] = key0 <= pos && key0 + 32 > k_lo;
-    if (live[i]) load_step<DT, POW2>(steps[i], kv, key0, k_lo, pos);
+    live[i] = key0 <= pos && (key0 + 32 > k_lo || key0 < st.keep);
+    int lo, hi;
+    step_bounds(key0, k_lo, pos, st.keep, lo, hi);
+    if (live[i]) load_step<DT, POW2>(steps[i], kv, key0, lo, hi);
   }
 #pragma unroll
   for (int i = 0; i < kDecodeWaveKeys / 32; ++i)
@@ -1040,7 +1082,7 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
   // the workspace holds the decode partials first, then the prefill partials
   float* prefill_ws = workspace ? workspace + attention_decode_workspace_floats(n_decode, nq, HD, max_decode_ctx) : nullptr;
   if (n_tiles > 0) {
-    if (staged_prefill(page_size)) {
+    if (staged_prefill(page_size) && st.keep == 0) {      // (kept first keys: the walk of the one-wave kernel knows them)
       int page_shift = 0;
       while ((1 << page_shift) < page_size) ++page_shift;
       const int splits = attention_prefill_splits(n_tiles, nq, nkv, HD, page_size, max_tile_ctx);

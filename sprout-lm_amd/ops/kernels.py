@@ -548,7 +548,7 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
     [nq], one logit per query head that joins the softmax's denominator without a key or value.  `mask_chunk`: a
     query sees only the keys of its own block of that many positions, counted from position 0.
     `keep_first`: a sequence's first keep_first keys stay visible to every later query beside its `window`; the
-    float32-arithmetic kernel on the vector units is the one that knows them, and such a call runs on it.
+    bfloat16 kernels and the float32-arithmetic kernel on the vector units know them, and such a call runs on those.
     `project`: (w_o [hidden, nq * hd], residual float32 [T, hidden]) of an output projection without bias
     that may be folded in: where the kernels take the step that way (one-query sequences only, bfloat16),
     residual += attention . w_o^T, `out` is left untouched and True is returned; otherwise False, and the
@@ -565,8 +565,8 @@ def attention(q: torch.Tensor, q_stride: int, k_pool: torch.Tensor, v_pool: torc
     keep_first = int(keep_first) if window else 0      # without a window every earlier key is visible anyway
     if keep_first < 0 or (keep_first and mask_chunk):
         raise KernelError("attention: kept first keys go with a window alone, and their number is not negative")
-    if keep_first:
-        kind = 2
+    if keep_first and (kind != 0 or q.dtype != torch.bfloat16):
+        kind = 2      # the bfloat16 kernels know kept first keys; of the float32-arithmetic kernels the one on the vector units
     for t, what in ((q, "q"), (out, "attention output")):
         _gpu(t, what)
     T = out.shape[0]
