@@ -201,6 +201,113 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(SsdArgs a) {
   }
 }
 
+// K numbers of a row in LDS as floats, eight or sixteen bytes at a time (the row starts at a multiple of 16 bytes).
+template <int K>
+__device__ __forceinline__ void lds_row(const bf16_t* p, float (&v)[K]) {
+#pragma unroll
+  for (int i = 0; i < K; i += 4) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p + i);
+    v[i] = __uint_as_float(w.x << 16);
+    v[i + 1] = __uint_as_float(w.x & 0xffff0000u);
+    v[i + 2] = __uint_as_float(w.y << 16);
+    v[i + 3] = __uint_as_float(w.y & 0xffff0000u);
+  }
+}
+template <int K>
+__device__ __forceinline__ void lds_row(const float* p, float (&v)[K]) {
+#pragma unroll
+  for (int i = 0; i < K; i += 4) {
+    const float4 w = *reinterpret_cast<const float4*>(p + i);
+    v[i] = w.x; v[i + 1] = w.y; v[i + 2] = w.z; v[i + 3] = w.w;
+  }
+}
+
+constexpr int kScanChunk = 64;      // tokens of a chunk where long portions are walked in chunks
+
+// MODE 1 and MODE 2 of the scan above for heads whose values come in whole 32s, so that a block's 32 columns lie in one
+// head: what the chunk's tokens share (B, C, the step sizes and decays, computed once per token and not once per lane)
+// and the block's columns of u and z are brought into LDS first, rows 8 * KPT wide with zeros behind the state's rows,
+// and the walk along the tokens reads LDS alone; lane rg holds the KPT neighbouring rows from rg * KPT on.
+template <typename T, int KPT, int MODE>
+__global__ __launch_bounds__(256) void ssd_chunk_kernel(SsdArgs a) {
+  constexpr int L = kScanChunk, NP = 8 * KPT;
+  extern __shared__ float4 lds_raw[];
+  float* Ds = reinterpret_cast<float*>(lds_raw);      // [L] step sizes, [L] decays
+  T* Bs = reinterpret_cast<T*>(Ds + 2 * L);           // [L][NP]
+  T* Cs = Bs + L * NP;                                // [L][NP]
+  T* Us = Cs + L * NP;                                // [L][32]
+  T* Zs = Us + L * 32;                                // [L][32]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int rg = lane & 7, pc = lane >> 3;
+  const int inner = a.heads * a.vdim, N = a.state_size;
+  const int s = blockIdx.y / a.chunks, ci = blockIdx.y % a.chunks;
+  const int col0 = blockIdx.x * 32, mine = wave * 8 + pc, col = col0 + mine;
+  const int n = col0 / a.vdim, p = col % a.vdim, g = n / (a.heads / a.groups);
+  const int q0 = a.q_start[s] + ci * L, len = min(L, a.q_len[s] - ci * L);
+  if (len <= 0) return;
+  const float rate = expf(a.a_log[n]), bias = a.dt_bias[n], skip = a.skip[n];
+  const T* proj = (const T*)a.proj;
+  const T* xbc = (const T*)a.xbc;
+  const int b_off = inner + g * N, c_off = inner + a.groups * N + g * N;
+  for (int i = threadIdx.x; i < len * NP; i += 256) {
+    const int tt = i / NP, r = i % NP;
+    const T* xr = xbc + size_t(q0 + tt) * a.xbc_stride;
+    Bs[i] = r < N ? xr[b_off + r] : from_float<T>(0.f);
+    if (MODE == 2) Cs[i] = r < N ? xr[c_off + r] : from_float<T>(0.f);
+  }
+  for (int i = threadIdx.x; i < len * 32; i += 256) {
+    const int tt = i >> 5, j = i & 31;
+    Us[i] = xbc[size_t(q0 + tt) * a.xbc_stride + col0 + j];
+    if (MODE == 2) Zs[i] = proj[size_t(q0 + tt) * a.proj_stride + a.z_off + col0 + j];
+  }
+  if (int(threadIdx.x) < len) {
+    const float d = softplus_of(to_float(proj[size_t(q0 + threadIdx.x) * a.proj_stride + a.dt_off + n]) + bias);
+    Ds[threadIdx.x] = d;
+    Ds[L + threadIdx.x] = expf(-rate * d);
+  }
+  float* S = a.scratch + ((size_t(blockIdx.y) * a.heads + n) * N) * a.vdim + p;
+  float st[KPT];
+#pragma unroll
+  for (int k = 0; k < KPT; ++k) {
+    const int r = rg * KPT + k;
+    st[k] = (MODE == 2 && r < N) ? S[size_t(r) * a.vdim] : 0.f;
+  }
+  __syncthreads();
+  float steps = 0.f;
+  for (int tt = 0; tt < len; ++tt) {
+    const float d = Ds[tt], decay = Ds[L + tt];
+    const float u = to_float(Us[tt * 32 + mine]);
+    const float du = d * u;
+    steps += d;
+    float b[KPT];
+    lds_row<KPT>(Bs + tt * NP + rg * KPT, b);
+    if (MODE == 1) {
+#pragma unroll
+      for (int k = 0; k < KPT; ++k) st[k] = fmaf(decay, st[k], du * b[k]);
+    } else {
+      float c[KPT];
+      lds_row<KPT>(Cs + tt * NP + rg * KPT, c);
+      float y = 0.f;
+#pragma unroll
+      for (int k = 0; k < KPT; ++k) {
+        st[k] = fmaf(decay, st[k], du * b[k]);
+        y = fmaf(st[k], c[k], y);
+      }
+      y += __shfl_xor(y, 1, 64);
+      y += __shfl_xor(y, 2, 64);
+      y += __shfl_xor(y, 4, 64);
+      if (rg == 0) a.out[size_t(q0 + tt) * inner + col] = fmaf(skip, u, y) * silu_of(to_float(Zs[tt * 32 + mine]));
+    }
+  }
+  if (MODE == 2) return;
+#pragma unroll
+  for (int k = 0; k < KPT; ++k) {
+    const int r = rg * KPT + k;
+    if (r < N) S[size_t(r) * a.vdim] = st[k];
+  }
+  if (p == 0 && rg == 0) a.step_sums[size_t(blockIdx.y) * a.heads + n] = steps;
+}
+
 // A thread a state element of a request: the chunks in turn.
 __global__ __launch_bounds__(256) void ssd_carry_kernel(SsdArgs a) {
   const int s = blockIdx.y;
@@ -487,7 +594,7 @@ extern "C" int sp_scale_rows(void* stream, int dtype, const void* x, const float
 }
 
 // Portions of more than kScanLong tokens are walked in chunks of kScanChunk.
-constexpr int kScanChunk = 64, kScanLong = 128;
+constexpr int kScanLong = 128;
 
 extern "C" long long sp_ssd_scan_scratch_floats(int heads, int vdim, int state_size, int n_seqs, int max_q_len) {
   if (max_q_len <= kScanLong || n_seqs <= 0) return 0;
@@ -543,11 +650,32 @@ extern "C" int sp_ssd_scan(void* stream, int dtype, const void* proj, long long 
   a.scratch = scratch;
   a.step_sums = scratch + size_t(n_seqs) * a.chunks * heads * state_size * vdim;
   const dim3 grid((inner + 31) / 32, n_seqs * a.chunks);
-  SP_SSD(1);
+  // heads of whole 32s of values whose chunk fits 64 KB of LDS: the kernels that bring a chunk into LDS first
+  const int kpt = state_size <= 32 ? 4 : state_size <= 64 ? 8 : state_size <= 128 ? 16 : 32;
+  const size_t element = dtype == kF32 ? 4 : 2;
+  const size_t lds = 2 * kScanChunk * sizeof(float) + 2 * size_t(kScanChunk) * (8 * kpt + 32) * element;
+  const bool staged = vdim % 32 == 0 && lds <= 64 * 1024;
+#define SP_SSD_CHUNK_MODE(KPT, MODE)                                                    \
+  do {                                                                                  \
+    if (dtype == kF32) ssd_chunk_kernel<float, KPT, MODE><<<grid, 256, lds, s>>>(a);    \
+    else ssd_chunk_kernel<bf16_t, KPT, MODE><<<grid, 256, lds, s>>>(a);                 \
+  } while (0)
+#define SP_SSD_CHUNK(MODE)                          \
+  do {                                              \
+    if (kpt == 4) SP_SSD_CHUNK_MODE(4, MODE);       \
+    else if (kpt == 8) SP_SSD_CHUNK_MODE(8, MODE);  \
+    else if (kpt == 16) SP_SSD_CHUNK_MODE(16, MODE);\
+    else SP_SSD_CHUNK_MODE(32, MODE);               \
+  } while (0)
+  if (staged) SP_SSD_CHUNK(1);
+  else SP_SSD(1);
   if (check_launch("sp_ssd_scan (chunks)")) return 1;
   ssd_carry_kernel<<<dim3((size_t(inner) * state_size + 255) / 256, n_seqs), 256, 0, s>>>(a);
   if (check_launch("sp_ssd_scan (carry)")) return 1;
-  SP_SSD(2);
+  if (staged) SP_SSD_CHUNK(2);
+  else SP_SSD(2);
+#undef SP_SSD_CHUNK
+#undef SP_SSD_CHUNK_MODE
 #undef SP_SSD
 #undef SP_SSD_MODE
   return check_launch("sp_ssd_scan (outputs)");
