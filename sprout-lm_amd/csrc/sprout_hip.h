@@ -302,11 +302,12 @@ long long sp_retention_scratch_floats(int heads, int dim, int vdim, int n_seqs, 
 // time per channel within each request; inputs before a request's share of the step come from its state rows
 // [slots, taps - 1, channels] (float32, oldest first; zeros in a fresh slot), which are left holding the request's last
 // taps - 1 inputs.  x [T, x_stride] from column x_off on, out [T, out_stride] from out_off on, both of `dtype`, not the
-// same memory; w [channels, taps] and bias (may be null) of w_dtype.  act 0: none, 1: SiLU.  taps 1: no state.
+// same memory; w TAP-major [taps, channels] and bias (may be null) of w_dtype.  act 0: none, 1: SiLU.  taps 1: no state.
+// max_q_len: the most tokens one request brings to the step (0: unknown); where it is 1, one launch does it all.
 int sp_short_conv(void* stream, int dtype, const void* x, long long x_stride, int x_off, int channels, int taps, int w_dtype,
                   const void* w, const void* bias, int act, int add_input, void* out, long long out_stride, int out_off,
                   const int32_t* q_start, const int32_t* q_len, const int32_t* seq_of_token, const int32_t* state_slots,
-                  float* state, int T, int n_seqs);
+                  float* state, int T, int n_seqs, int max_q_len);
 // out [T, parts * size] = x / sqrt(mean over each part of x^2 + eps) * w, every row in `parts` equal parts, x float32.
 int sp_group_rmsnorm(void* stream, const float* x, int w_dtype, const void* w, float eps, int out_dtype, void* out, int T,
                      int parts, int size);

@@ -33,6 +33,7 @@ struct ConvArgs {
 };
 
 // A thread a (token, channel): the taps in their order, inputs before the request's share of the step from its state rows.
+// The weights lie tap-major, [taps][channels].
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void short_conv_kernel(ConvArgs a) {
   const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
@@ -40,16 +41,94 @@ __global__ __launch_bounds__(256) void short_conv_kernel(ConvArgs a) {
   const int s = a.seq_of_token[t];
   const int j = t - a.q_start[s], keep = a.taps - 1;
   const T* x = (const T*)a.x + a.x_off + c;
-  const TW* w = (const TW*)a.w + size_t(c) * a.taps;
+  const TW* w = (const TW*)a.w + c;
   const float* rows = keep ? a.state + size_t(a.state_slots[s]) * keep * a.channels + c : nullptr;
   float acc = a.bias ? to_float(((const TW*)a.bias)[c]) : 0.f;
   for (int tap = 0; tap < a.taps; ++tap) {
     const int back = keep - tap;
     const float v = j - back >= 0 ? to_float(x[size_t(t - back) * a.x_stride]) : rows[size_t(keep + j - back) * a.channels];
-    acc = fmaf(to_float(w[tap]), v, acc);
+    acc = fmaf(to_float(w[size_t(tap) * a.channels]), v, acc);
   }
   if (a.act == 1) acc = silu_of(acc);
   if (a.add_input) acc += to_float(x[size_t(t) * a.x_stride]);
+  ((T*)a.out)[size_t(t) * a.out_stride + a.out_off + c] = from_float<T>(acc);
+}
+
+__device__ __forceinline__ void unpack8(const uint4& raw, float (&v)[8]) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __uint_as_float(w[i] << 16);
+    v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+// The same for bfloat16 rows and weights whose channels come in whole eights at 16 bytes: a thread eight neighbouring
+// channels of a token, sixteen bytes a load.  The sums run in the taps' order, as above.
+__global__ __launch_bounds__(256) void short_conv_eights_kernel(ConvArgs a) {
+  const int t = blockIdx.x, c = 8 * (blockIdx.y * 256 + threadIdx.x);
+  if (c >= a.channels) return;
+  const int s = a.seq_of_token[t];
+  const int j = t - a.q_start[s], keep = a.taps - 1;
+  const bf16_t* x = (const bf16_t*)a.x + a.x_off + c;
+  const bf16_t* w = (const bf16_t*)a.w + c;
+  const float* rows = keep ? a.state + size_t(a.state_slots[s]) * keep * a.channels + c : nullptr;
+  float acc[8], v[8], wt[8];
+  if (a.bias) unpack8(*reinterpret_cast<const uint4*>((const bf16_t*)a.bias + c), acc);
+  else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  }
+  for (int tap = 0; tap < a.taps; ++tap) {
+    const int back = keep - tap;
+    if (j - back >= 0) {
+      unpack8(*reinterpret_cast<const uint4*>(x + size_t(t - back) * a.x_stride), v);
+    } else {
+      const float4* r = reinterpret_cast<const float4*>(rows + size_t(keep + j - back) * a.channels);
+      const float4 lo = r[0], hi = r[1];
+      v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+    }
+    unpack8(*reinterpret_cast<const uint4*>(w + size_t(tap) * a.channels), wt);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = fmaf(wt[i], v[i], acc[i]);
+  }
+  if (a.act == 1) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = silu_of(acc[i]);
+  }
+  if (a.add_input) {
+    unpack8(*reinterpret_cast<const uint4*>(x + size_t(t) * a.x_stride), v);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += v[i];
+  }
+  uint4 packed;
+  packed.x = uint32_t(f32_to_bf16_bits(acc[0])) | uint32_t(f32_to_bf16_bits(acc[1])) << 16;
+  packed.y = uint32_t(f32_to_bf16_bits(acc[2])) | uint32_t(f32_to_bf16_bits(acc[3])) << 16;
+  packed.z = uint32_t(f32_to_bf16_bits(acc[4])) | uint32_t(f32_to_bf16_bits(acc[5])) << 16;
+  packed.w = uint32_t(f32_to_bf16_bits(acc[6])) | uint32_t(f32_to_bf16_bits(acc[7])) << 16;
+  *reinterpret_cast<uint4*>((bf16_t*)a.out + size_t(t) * a.out_stride + a.out_off + c) = packed;
+}
+
+// A step in which every request brings one token: the thread that owns a (request, channel) convolves and moves the
+// state rows up itself, in one launch.  The sum runs in the taps' order, as above.
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void short_conv_single_kernel(ConvArgs a) {
+  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= a.channels) return;
+  const int s = a.seq_of_token[t], keep = a.taps - 1;
+  const float x = to_float(((const T*)a.x)[size_t(t) * a.x_stride + a.x_off + c]);
+  const TW* w = (const TW*)a.w + c;
+  float* rows = a.state + size_t(a.state_slots[s]) * keep * a.channels + c;
+  float acc = a.bias ? to_float(((const TW*)a.bias)[c]) : 0.f;
+  for (int tap = 0; tap < keep; ++tap) {
+    const float v = rows[size_t(tap) * a.channels];
+    acc = fmaf(to_float(w[size_t(tap) * a.channels]), v, acc);
+    if (tap > 0) rows[size_t(tap - 1) * a.channels] = v;
+  }
+  rows[size_t(keep - 1) * a.channels] = x;
+  acc = fmaf(to_float(w[size_t(keep) * a.channels]), x, acc);
+  if (a.act == 1) acc = silu_of(acc);
+  if (a.add_input) acc += x;
   ((T*)a.out)[size_t(t) * a.out_stride + a.out_off + c] = from_float<T>(acc);
 }
 
@@ -249,11 +328,22 @@ __global__ __launch_bounds__(256) void ssd_chunk_kernel(SsdArgs a) {
   const T* proj = (const T*)a.proj;
   const T* xbc = (const T*)a.xbc;
   const int b_off = inner + g * N, c_off = inner + a.groups * N + g * N;
-  for (int i = threadIdx.x; i < len * NP; i += 256) {
-    const int tt = i / NP, r = i % NP;
-    const T* xr = xbc + size_t(q0 + tt) * a.xbc_stride;
-    Bs[i] = r < N ? xr[b_off + r] : from_float<T>(0.f);
-    if (MODE == 2) Cs[i] = r < N ? xr[c_off + r] : from_float<T>(0.f);
+  if (sizeof(T) == 2 && N == NP && (a.xbc_stride & 7) == 0 && (b_off & 7) == 0 && (c_off & 7) == 0 &&
+      (reinterpret_cast<uintptr_t>(xbc) & 15) == 0) {
+    // rows of whole eights at 16 bytes: eight numbers a load
+    for (int i = threadIdx.x; i < len * (NP / 8); i += 256) {
+      const int tt = i / (NP / 8), r = 8 * (i % (NP / 8));
+      const T* xr = xbc + size_t(q0 + tt) * a.xbc_stride;
+      *reinterpret_cast<uint4*>(Bs + tt * NP + r) = *reinterpret_cast<const uint4*>(xr + b_off + r);
+      if (MODE == 2) *reinterpret_cast<uint4*>(Cs + tt * NP + r) = *reinterpret_cast<const uint4*>(xr + c_off + r);
+    }
+  } else {
+    for (int i = threadIdx.x; i < len * NP; i += 256) {
+      const int tt = i / NP, r = i % NP;
+      const T* xr = xbc + size_t(q0 + tt) * a.xbc_stride;
+      Bs[i] = r < N ? xr[b_off + r] : from_float<T>(0.f);
+      if (MODE == 2) Cs[i] = r < N ? xr[c_off + r] : from_float<T>(0.f);
+    }
   }
   for (int i = threadIdx.x; i < len * 32; i += 256) {
     const int tt = i >> 5, j = i & 31;
@@ -420,6 +510,83 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SelArgs a) {
   }
 }
 
+// MODE 1 and MODE 2 of the scan above with the chunk in LDS: the step sizes (their softplus taken once per token and
+// channel, not once per lane), the block's columns of u and z, and B and C as floats in rows 4 * KPT wide with zeros behind
+// the state's numbers; lane ng holds the KPT neighbouring states from ng * KPT on.
+template <typename T, int KPT, int MODE>
+__global__ __launch_bounds__(256) void selective_chunk_kernel(SelArgs a) {
+  constexpr int L = kScanChunk, NP = 4 * KPT;
+  extern __shared__ float4 lds_raw[];
+  float* Ds = reinterpret_cast<float*>(lds_raw);      // [L][64]
+  float* BCs = Ds + L * 64;                           // [L][2][NP]
+  T* Us = reinterpret_cast<T*>(BCs + L * 2 * NP);     // [L][64]
+  T* Zs = Us + L * 64;                                // [L][64]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int ng = lane & 3, cc = lane >> 2, mine = wave * 16 + cc;
+  const int N = a.state_size;
+  const int s = blockIdx.y / a.chunks, ci = blockIdx.y % a.chunks;
+  const int c0 = blockIdx.x * 64;
+  int c = c0 + mine;
+  const bool live = c < a.inner;
+  if (!live) c = a.inner - 1;
+  const int q0 = a.q_start[s] + ci * L, len = min(L, a.q_len[s] - ci * L);
+  if (len <= 0) return;
+  for (int i = threadIdx.x; i < len * 64; i += 256) {
+    const int tt = i >> 6, ch = min(c0 + (i & 63), a.inner - 1);
+    const size_t t = size_t(q0 + tt);
+    Ds[i] = softplus_of(a.dt[t * a.inner + ch]);
+    Us[i] = ((const T*)a.u)[t * a.u_stride + a.u_off + ch];
+    if (MODE == 2) Zs[i] = ((const T*)a.z)[t * a.z_stride + a.z_off + ch];
+  }
+  for (int i = threadIdx.x; i < len * 2 * NP; i += 256) {
+    const int tt = i / (2 * NP), r = i % (2 * NP), which = r / NP, nn = r % NP;
+    BCs[i] = nn < N ? to_float(((const T*)a.bc)[size_t(q0 + tt) * a.bc_stride + a.bc_off + which * N + nn]) : 0.f;
+  }
+  float* S = a.scratch + (size_t(blockIdx.y) * a.inner + c) * N;
+  float st[KPT], ak[KPT];
+#pragma unroll
+  for (int k = 0; k < KPT; ++k) {
+    const int n = ng * KPT + k;
+    st[k] = (MODE == 2 && n < N) ? S[n] : 0.f;
+    ak[k] = n < N ? a.a[size_t(c) * N + n] : 0.f;
+  }
+  const float skip = a.skip[c];
+  __syncthreads();
+  float steps = 0.f;
+  for (int tt = 0; tt < len; ++tt) {
+    const float d = Ds[tt * 64 + mine];
+    const float u = to_float(Us[tt * 64 + mine]);
+    const float du = d * u;
+    steps += d;
+    float b[KPT];
+    lds_row<KPT>(BCs + tt * 2 * NP + ng * KPT, b);
+    if (MODE == 1) {
+#pragma unroll
+      for (int k = 0; k < KPT; ++k) st[k] = fmaf(expf(d * ak[k]), st[k], du * b[k]);
+    } else {
+      float cv[KPT];
+      lds_row<KPT>(BCs + tt * 2 * NP + NP + ng * KPT, cv);
+      float y = 0.f;
+#pragma unroll
+      for (int k = 0; k < KPT; ++k) {
+        st[k] = fmaf(expf(d * ak[k]), st[k], du * b[k]);
+        y = fmaf(st[k], cv[k], y);
+      }
+      y += __shfl_xor(y, 1, 64);
+      y += __shfl_xor(y, 2, 64);
+      if (ng == 0 && live)
+        ((T*)a.out)[size_t(q0 + tt) * a.inner + c] = from_float<T>(fmaf(skip, u, y) * silu_of(to_float(Zs[tt * 64 + mine])));
+    }
+  }
+  if (MODE == 2 || !live) return;
+#pragma unroll
+  for (int k = 0; k < KPT; ++k) {
+    const int n = ng * KPT + k;
+    if (n < N) S[n] = st[k];
+  }
+  if (ng == 0) a.step_sums[size_t(blockIdx.y) * a.inner + c] = steps;
+}
+
 __global__ __launch_bounds__(256) void selective_carry_kernel(SelArgs a) {
   const int s = blockIdx.y;
   const size_t per_request = size_t(a.inner) * a.state_size;
@@ -534,7 +701,8 @@ using namespace sprout;
 extern "C" int sp_short_conv(void* stream, int dtype, const void* x, long long x_stride, int x_off, int channels, int taps,
                              int w_dtype, const void* w, const void* bias, int act, int add_input, void* out,
                              long long out_stride, int out_off, const int32_t* q_start, const int32_t* q_len,
-                             const int32_t* seq_of_token, const int32_t* state_slots, float* state, int T, int n_seqs) {
+                             const int32_t* seq_of_token, const int32_t* state_slots, float* state, int T, int n_seqs,
+                             int max_q_len) {
   SP_REQUIRE(dtype == kF32 || dtype == kBF16, "sp_short_conv: unsupported dtype %d", dtype);
   SP_REQUIRE(w_dtype == dtype || w_dtype == kF32, "sp_short_conv: weights of dtype %d beside rows of dtype %d", w_dtype, dtype);
   SP_REQUIRE(channels > 0 && taps > 0 && taps <= 64 && T >= 0 && n_seqs >= 0, "sp_short_conv: bad sizes (%d channels, %d taps)", channels, taps);
@@ -548,7 +716,17 @@ extern "C" int sp_short_conv(void* stream, int dtype, const void* x, long long x
                       q_start, q_len, seq_of_token, state_slots, state};
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(T, (channels + 255) / 256);
-  if (dtype == kF32) short_conv_kernel<float, float><<<grid, 256, 0, s>>>(a);
+  if (max_q_len == 1 && taps > 1) {      // single tokens: one launch convolves and moves the state rows up
+    if (dtype == kF32) short_conv_single_kernel<float, float><<<grid, 256, 0, s>>>(a);
+    else if (w_dtype == kF32) short_conv_single_kernel<bf16_t, float><<<grid, 256, 0, s>>>(a);
+    else short_conv_single_kernel<bf16_t, bf16_t><<<grid, 256, 0, s>>>(a);
+    return check_launch("sp_short_conv (single tokens)");
+  }
+  const auto at16 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  const bool eights = dtype == kBF16 && w_dtype == kBF16 && T >= 64 && channels % 8 == 0 && x_off % 8 == 0 && out_off % 8 == 0 &&
+                      x_stride % 8 == 0 && out_stride % 8 == 0 && at16(x) && at16(out) && at16(w) && at16(bias) && at16(state);
+  if (eights) short_conv_eights_kernel<<<dim3(T, (channels / 8 + 255) / 256), 256, 0, s>>>(a);
+  else if (dtype == kF32) short_conv_kernel<float, float><<<grid, 256, 0, s>>>(a);
   else if (w_dtype == kF32) short_conv_kernel<bf16_t, float><<<grid, 256, 0, s>>>(a);
   else short_conv_kernel<bf16_t, bf16_t><<<grid, 256, 0, s>>>(a);
   if (check_launch("sp_short_conv")) return 1;
@@ -721,11 +899,31 @@ extern "C" int sp_selective_scan(void* stream, int dtype, const void* u, long lo
   args.scratch = scratch;
   args.step_sums = scratch + size_t(n_seqs) * args.chunks * inner * state_size;
   const dim3 grid((inner + 63) / 64, n_seqs * args.chunks);
-  SP_SEL(1);
+  // where a chunk fits 64 KB of LDS: the kernels that bring it there first
+  const int kpt = state_size <= 16 ? 4 : state_size <= 32 ? 8 : state_size <= 64 ? 16 : state_size <= 128 ? 32 : 64;
+  const size_t lds = size_t(kScanChunk) * (64 + 8 * kpt) * sizeof(float) + 2 * size_t(kScanChunk) * 64 * (dtype == kF32 ? 4 : 2);
+  const bool staged = lds <= 64 * 1024;
+#define SP_SEL_CHUNK_MODE(KPT, MODE)                                                            \
+  do {                                                                                          \
+    if (dtype == kF32) selective_chunk_kernel<float, KPT, MODE><<<grid, 256, lds, s>>>(args);   \
+    else selective_chunk_kernel<bf16_t, KPT, MODE><<<grid, 256, lds, s>>>(args);                \
+  } while (0)
+#define SP_SEL_CHUNK(MODE)                           \
+  do {                                               \
+    if (kpt == 4) SP_SEL_CHUNK_MODE(4, MODE);        \
+    else if (kpt == 8) SP_SEL_CHUNK_MODE(8, MODE);   \
+    else if (kpt == 16) SP_SEL_CHUNK_MODE(16, MODE); \
+    else SP_SEL_CHUNK_MODE(32, MODE);                \
+  } while (0)
+  if (staged) SP_SEL_CHUNK(1);
+  else SP_SEL(1);
   if (check_launch("sp_selective_scan (chunks)")) return 1;
   selective_carry_kernel<<<dim3((size_t(inner) * state_size + 255) / 256, n_seqs), 256, 0, s>>>(args);
   if (check_launch("sp_selective_scan (carry)")) return 1;
-  SP_SEL(2);
+  if (staged) SP_SEL_CHUNK(2);
+  else SP_SEL(2);
+#undef SP_SEL_CHUNK
+#undef SP_SEL_CHUNK_MODE
 #undef SP_SEL
 #undef SP_SEL_MODE
   return check_launch("sp_selective_scan (outputs)");

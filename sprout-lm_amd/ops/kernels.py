@@ -840,17 +840,18 @@ def _step_ints(q_start, q_len, state_slots, n_seqs: int, seq_of_token=None, T: i
 
 def short_conv(x: torch.Tensor, x_off: int, channels: int, taps: int, w: torch.Tensor, bias, out: torch.Tensor, out_off: int,
                q_start, q_len, seq_of_token, state_slots, n_seqs: int, state, act: str | None = None,
-               add_input: bool = False) -> None:
+               add_input: bool = False, max_q_len: int = 0) -> None:
     """The causal convolution of sp_short_conv (sprout_hip.h) on columns x_off .. x_off + channels of a step's rows `x`, into
-    columns out_off .. of `out` (another tensor of the same dtype).  `state`: float32 [slots, taps - 1, channels], the
-    requests' last inputs, read and left behind; None with one tap.  `act`: None or "silu"."""
+    columns out_off .. of `out` (another tensor of the same dtype).  `w`: TAP-major [taps, channels].  `state`: float32
+    [slots, taps - 1, channels], the requests' last inputs, read and left behind; None with one tap.  `act`: None or
+    "silu".  `max_q_len`: the most tokens one request brings (0: unknown)."""
     _gpu(x, "convolution input"); _gpu(out, "convolution output"); _gpu(w, "convolution weights")
     T = out.shape[0]
     if x.dim() != 2 or out.dim() != 2 or x.shape[0] < T or x.dtype != out.dtype or x_off + channels > x.shape[1] \
             or out_off + channels > out.shape[1] or x.data_ptr() == out.data_ptr():
         raise KernelError(f"short_conv: rows {tuple(x.shape)} {x.dtype} and {tuple(out.shape)} {out.dtype} do not fit {channels} channels")
-    if tuple(w.shape) != (channels, taps) or not w.is_contiguous() or (bias is not None and (bias.numel() != channels or bias.dtype != w.dtype)):
-        raise KernelError(f"short_conv: weights must be [{channels}, {taps}] with a bias of {channels}")
+    if tuple(w.shape) != (taps, channels) or not w.is_contiguous() or (bias is not None and (bias.numel() != channels or bias.dtype != w.dtype)):
+        raise KernelError(f"short_conv: weights must be tap-major [{taps}, {channels}] with a bias of {channels}")
     if act not in (None, "silu"):
         raise KernelError(f"short_conv: no activation {act!r}")
     _step_ints(q_start, q_len, state_slots, n_seqs, seq_of_token, T)
@@ -864,7 +865,7 @@ def short_conv(x: torch.Tensor, x_off: int, channels: int, taps: int, w: torch.T
                                   _code(w, "convolution weights"), w.data_ptr(), _ptr(bias), 1 if act == "silu" else 0,
                                   int(bool(add_input)), out.data_ptr(), out.stride(0), out_off, q_start.data_ptr(),
                                   q_len.data_ptr(), seq_of_token.data_ptr(), state_slots.data_ptr(),
-                                  state.data_ptr() if taps > 1 else None, T, n_seqs))
+                                  state.data_ptr() if taps > 1 else None, T, n_seqs, int(max_q_len)))
 
 
 def group_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor, parts: int) -> None:

@@ -82,7 +82,7 @@ def _declare(lib):
         "sp_route_combine": [c_void, c_void, c_void, c_void, c_int, c_void, c_int, c_int],
         "sp_route_sigmoid": [c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_int, c_void, c_void, c_void, c_void],
         "sp_short_conv": [c_void, c_int, c_void, c_i64, c_int, c_int, c_int, c_int, c_void, c_void, c_int, c_int, c_void, c_i64,
-                          c_int, c_void, c_void, c_void, c_void, c_void, c_int, c_int],
+                          c_int, c_void, c_void, c_void, c_void, c_void, c_int, c_int, c_int],
         "sp_group_rmsnorm": [c_void, c_void, c_int, c_void, c_float, c_int, c_void, c_int, c_int, c_int],
         "sp_activation": [c_void, c_int, c_void, c_i64, c_int],
         "sp_scale_rows": [c_void, c_int, c_void, c_void, c_int, c_void, c_int, c_int],

@@ -39,12 +39,12 @@ class ShortConv(Part):
 
     def bind(self, tensors):
         self.w = tensors
-        self.weight = tensors[self.tensor].contiguous()
+        self.weight = tensors[self.tensor].t().contiguous()      # tap-major: neighbouring channels lie together
         self.b = tensors[self.bias].contiguous() if self.bias is not None else None
 
     def forward(self, ctx, x, out, cache, x_off: int = 0, out_off: int = 0):
         """out[:, out_off : out_off + channels] = conv(x[:, x_off : x_off + channels]); x and out are different tensors."""
         ops.short_conv(x, x_off, self.channels, self.taps, self.weight, self.b, out, out_off, ctx.q_start, ctx.q_len,
                        ctx.seq_of_token, ctx.state_slots, ctx.n_seqs, cache.state if self.taps > 1 else None,
-                       act=self.activation, add_input=self.residual)
+                       act=self.activation, add_input=self.residual, max_q_len=ctx.max_q_len)
         return out
