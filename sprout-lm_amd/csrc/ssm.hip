@@ -6,6 +6,8 @@
 // state_slots (one entry per request of the step) say where a request's tokens are and which row of the state tensors is
 // its own.  A kernel reads the state as the step before left it and leaves it for the next one, so a portion of a prompt
 // and a single decoded token are the same call.
+#include <type_traits>
+
 #include "common.h"
 #include "sprout_hip.h"
 
@@ -198,8 +200,9 @@ struct SsdArgs {
   float* state;
   float* out;
   int chunk, chunks;           // tokens a chunk, chunks a request (the longest portion's), where portions are walked in chunks
-  float* scratch;              // [requests * chunks, heads, state, vdim]
+  float* scratch;              // [requests * chunks, heads, state, vdim]; by_column: [requests * chunks, heads, vdim, state]
   float* step_sums;            // [requests * chunks, heads]
+  int by_column;               // the scratch holds a column's state rows together (what a lane of the LDS kernels owns)
 };
 
 // A block per request and 32 columns of the heads' values; a column's state rows are shared out over 8 neighbouring lanes
@@ -304,18 +307,24 @@ __device__ __forceinline__ void lds_row(const float* p, float (&v)[K]) {
 constexpr int kScanChunk = 64;      // tokens of a chunk where long portions are walked in chunks
 
 // MODE 1 and MODE 2 of the scan above for heads whose values come in whole 32s, so that a block's 32 columns lie in one
-// head: what the chunk's tokens share (B, C, the step sizes and decays, computed once per token and not once per lane)
-// and the block's columns of u and z are brought into LDS first, rows 8 * KPT wide with zeros behind the state's rows,
-// and the walk along the tokens reads LDS alone; lane rg holds the KPT neighbouring rows from rg * KPT on.
+// head: what the chunk's tokens share (B and C as floats, the step sizes and decays, computed once per token and not once
+// per lane) and the block's columns of u and z are brought into LDS first, rows 8 * KPT wide with zeros behind the
+// state's rows, and the walk along the tokens reads LDS alone; lane rg holds the KPT neighbouring rows from rg * KPT on.
+// The kernels are bound by their vector instructions (a multiply-add per state element and token is what the design
+// asks for), so MODE 1 does not walk the recurrence: what a chunk adds to a state of zeros is
+// sum_t w_t u_t B_t with w_t = d_t exp(-rate * (the step sizes after t)), one multiply-add per element and token.
 template <typename T, int KPT, int MODE>
 __global__ __launch_bounds__(256) void ssd_chunk_kernel(SsdArgs a) {
   constexpr int L = kScanChunk, NP = 8 * KPT;
   extern __shared__ float4 lds_raw[];
-  float* Ds = reinterpret_cast<float*>(lds_raw);      // [L] step sizes, [L] decays
-  T* Bs = reinterpret_cast<T*>(Ds + 2 * L);           // [L][NP]
-  T* Cs = Bs + L * NP;                                // [L][NP]
-  T* Us = Cs + L * NP;                                // [L][32]
-  T* Zs = Us + L * 32;                                // [L][32]
+  // B and C in LDS: floats for MODE 1, whose one multiply-add per element leaves no room for conversions; as they are
+  // stored for MODE 2, which waits for LDS more than for its arithmetic when the rows are twice as long
+  using TL = typename std::conditional<MODE == 1, float, T>::type;
+  float* Ds = reinterpret_cast<float*>(lds_raw);      // [L] step sizes, [L] decays (MODE 2) or weights w_t (MODE 1)
+  TL* Bs = reinterpret_cast<TL*>(Ds + 2 * L);         // [L][NP]
+  TL* Cs = Bs + L * NP;                               // [L][NP], MODE 2 only
+  T* Us = reinterpret_cast<T*>(MODE == 2 ? Cs + L * NP : Cs);      // [L][32]
+  T* Zs = Us + L * 32;                                // [L][32], MODE 2 only
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rg = lane & 7, pc = lane >> 3;
   const int inner = a.heads * a.vdim, N = a.state_size;
@@ -334,15 +343,23 @@ __global__ __launch_bounds__(256) void ssd_chunk_kernel(SsdArgs a) {
     for (int i = threadIdx.x; i < len * (NP / 8); i += 256) {
       const int tt = i / (NP / 8), r = 8 * (i % (NP / 8));
       const T* xr = xbc + size_t(q0 + tt) * a.xbc_stride;
-      *reinterpret_cast<uint4*>(Bs + tt * NP + r) = *reinterpret_cast<const uint4*>(xr + b_off + r);
-      if (MODE == 2) *reinterpret_cast<uint4*>(Cs + tt * NP + r) = *reinterpret_cast<const uint4*>(xr + c_off + r);
+      if (MODE == 1) {
+        float v[8];
+        unpack8(*reinterpret_cast<const uint4*>(xr + b_off + r), v);
+        float4* to = reinterpret_cast<float4*>(Bs + tt * NP + r);
+        to[0] = make_float4(v[0], v[1], v[2], v[3]);
+        to[1] = make_float4(v[4], v[5], v[6], v[7]);
+      } else {
+        *reinterpret_cast<uint4*>(Bs + tt * NP + r) = *reinterpret_cast<const uint4*>(xr + b_off + r);
+        *reinterpret_cast<uint4*>(Cs + tt * NP + r) = *reinterpret_cast<const uint4*>(xr + c_off + r);
+      }
     }
   } else {
     for (int i = threadIdx.x; i < len * NP; i += 256) {
       const int tt = i / NP, r = i % NP;
       const T* xr = xbc + size_t(q0 + tt) * a.xbc_stride;
-      Bs[i] = r < N ? xr[b_off + r] : from_float<T>(0.f);
-      if (MODE == 2) Cs[i] = r < N ? xr[c_off + r] : from_float<T>(0.f);
+      Bs[i] = from_float<TL>(r < N ? to_float(xr[b_off + r]) : 0.f);
+      if (MODE == 2) Cs[i] = from_float<TL>(r < N ? to_float(xr[c_off + r]) : 0.f);
     }
   }
   for (int i = threadIdx.x; i < len * 32; i += 256) {
@@ -353,49 +370,93 @@ __global__ __launch_bounds__(256) void ssd_chunk_kernel(SsdArgs a) {
   if (int(threadIdx.x) < len) {
     const float d = softplus_of(to_float(proj[size_t(q0 + threadIdx.x) * a.proj_stride + a.dt_off + n]) + bias);
     Ds[threadIdx.x] = d;
-    Ds[L + threadIdx.x] = expf(-rate * d);
+    if (MODE == 2) Ds[L + threadIdx.x] = expf(-rate * d);
   }
-  float* S = a.scratch + ((size_t(blockIdx.y) * a.heads + n) * N) * a.vdim + p;
+  // a column's state rows lie together in the scratch: a lane's KPT rows are one run of memory
+  float* S = a.scratch + ((size_t(blockIdx.y) * a.heads + n) * a.vdim + p) * N + rg * KPT;
   float st[KPT];
 #pragma unroll
-  for (int k = 0; k < KPT; ++k) {
-    const int r = rg * KPT + k;
-    st[k] = (MODE == 2 && r < N) ? S[size_t(r) * a.vdim] : 0.f;
-  }
-  __syncthreads();
-  float steps = 0.f;
-  for (int tt = 0; tt < len; ++tt) {
-    const float d = Ds[tt], decay = Ds[L + tt];
-    const float u = to_float(Us[tt * 32 + mine]);
-    const float du = d * u;
-    steps += d;
-    float b[KPT];
-    lds_row<KPT>(Bs + tt * NP + rg * KPT, b);
-    if (MODE == 1) {
+  for (int k = 0; k < KPT; ++k) st[k] = 0.f;
+  if (MODE == 2) {
+    if (N == NP) {
 #pragma unroll
-      for (int k = 0; k < KPT; ++k) st[k] = fmaf(decay, st[k], du * b[k]);
-    } else {
-      float c[KPT];
-      lds_row<KPT>(Cs + tt * NP + rg * KPT, c);
-      float y = 0.f;
-#pragma unroll
-      for (int k = 0; k < KPT; ++k) {
-        st[k] = fmaf(decay, st[k], du * b[k]);
-        y = fmaf(st[k], c[k], y);
+      for (int k = 0; k < KPT; k += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(S + k);
+        st[k] = v.x; st[k + 1] = v.y; st[k + 2] = v.z; st[k + 3] = v.w;
       }
-      y += __shfl_xor(y, 1, 64);
-      y += __shfl_xor(y, 2, 64);
-      y += __shfl_xor(y, 4, 64);
-      if (rg == 0) a.out[size_t(q0 + tt) * inner + col] = fmaf(skip, u, y) * silu_of(to_float(Zs[tt * 32 + mine]));
+    } else {
+#pragma unroll
+      for (int k = 0; k < KPT; ++k)
+        if (rg * KPT + k < N) st[k] = S[k];
     }
   }
-  if (MODE == 2) return;
+  __syncthreads();
+  if (MODE == 1) {
+    // w_t = d_t exp(-rate * (d_(t+1) + ... + d_(len-1))): every token's weight in the chunk's last state
+    if (int(threadIdx.x) < len) {
+      float after = 0.f;
+      for (int t2 = len - 1; t2 > int(threadIdx.x); --t2) after += Ds[t2];
+      Ds[L + threadIdx.x] = Ds[threadIdx.x] * expf(-rate * after);
+      if (threadIdx.x == 0 && blockIdx.x * 32 == n * a.vdim) a.step_sums[size_t(blockIdx.y) * a.heads + n] = after + Ds[0];
+    }
+    __syncthreads();
+    for (int tt = 0; tt < len; ++tt) {
+      const float wu = Ds[L + tt] * to_float(Us[tt * 32 + mine]);
+      float b[KPT];
+      lds_row<KPT>(Bs + tt * NP + rg * KPT, b);
 #pragma unroll
-  for (int k = 0; k < KPT; ++k) {
-    const int r = rg * KPT + k;
-    if (r < N) S[size_t(r) * a.vdim] = st[k];
+      for (int k = 0; k < KPT; ++k) st[k] = fmaf(wu, b[k], st[k]);
+    }
+  } else {
+    // eight tokens at a time: a lane's share of each token's output, then the eight lanes of a column exchange them so that
+    // lane rg ends with the whole sum of token rg (three exchanges of 4, 2 and 1 numbers instead of three of 8), and
+    // every lane finishes and stores one token's output
+    for (int t0 = 0; t0 < len; t0 += 8) {
+      float part[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int tt = min(t0 + i, len - 1);
+        const bool real = t0 + i < len;
+        const float d = Ds[tt], decay = real ? Ds[L + tt] : 1.f;
+        const float du = real ? d * to_float(Us[tt * 32 + mine]) : 0.f;
+        float b[KPT], c[KPT];
+        lds_row<KPT>(Bs + tt * NP + rg * KPT, b);
+        lds_row<KPT>(Cs + tt * NP + rg * KPT, c);
+        float y = 0.f;
+#pragma unroll
+        for (int k = 0; k < KPT; ++k) {
+          st[k] = fmaf(decay, st[k], du * b[k]);
+          y = fmaf(st[k], c[k], y);
+        }
+        part[i] = y;
+      }
+      float four[4], two[2];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float keep = (rg & 4) ? part[i + 4] : part[i], give = (rg & 4) ? part[i] : part[i + 4];
+        four[i] = keep + __shfl_xor(give, 4, 64);
+      }
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const float keep = (rg & 2) ? four[i + 2] : four[i], give = (rg & 2) ? four[i] : four[i + 2];
+        two[i] = keep + __shfl_xor(give, 2, 64);
+      }
+      const float keep = (rg & 1) ? two[1] : two[0], give = (rg & 1) ? two[0] : two[1];
+      const float y = keep + __shfl_xor(give, 1, 64);
+      const int tt = t0 + rg;
+      if (tt < len)
+        a.out[size_t(q0 + tt) * inner + col] = fmaf(skip, to_float(Us[tt * 32 + mine]), y) * silu_of(to_float(Zs[tt * 32 + mine]));
+    }
+    return;
   }
-  if (p == 0 && rg == 0) a.step_sums[size_t(blockIdx.y) * a.heads + n] = steps;
+  if (N == NP) {
+#pragma unroll
+    for (int k = 0; k < KPT; k += 4) *reinterpret_cast<float4*>(S + k) = make_float4(st[k], st[k + 1], st[k + 2], st[k + 3]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < KPT; ++k)
+      if (rg * KPT + k < N) S[k] = st[k];
+  }
 }
 
 // A thread a state element of a request: the chunks in turn.
@@ -408,7 +469,13 @@ __global__ __launch_bounds__(256) void ssd_carry_kernel(SsdArgs a) {
   if (L <= 0) return;
   const int n = int(e / per_head), used = (L + a.chunk - 1) / a.chunk;
   const float rate = expf(a.a_log[n]);
-  float* mine = a.state + size_t(a.state_slots[s]) * per_request + e;
+  // e counts the scratch's elements; the request's own rows lie [head][state][vdim]
+  size_t own = e;
+  if (a.by_column) {
+    const size_t in_head = e % per_head;
+    own = size_t(n) * per_head + (in_head % a.state_size) * a.vdim + in_head / a.state_size;
+  }
+  float* mine = a.state + size_t(a.state_slots[s]) * per_request + own;
   float S = *mine;
   for (int c = 0; c < used; ++c) {
     const size_t number = size_t(s) * a.chunks + c;
@@ -548,34 +615,55 @@ __global__ __launch_bounds__(256) void selective_chunk_kernel(SelArgs a) {
   for (int k = 0; k < KPT; ++k) {
     const int n = ng * KPT + k;
     st[k] = (MODE == 2 && n < N) ? S[n] : 0.f;
-    ak[k] = n < N ? a.a[size_t(c) * N + n] : 0.f;
+    ak[k] = n < N ? a.a[size_t(c) * N + n] * 1.4426950408889634f : 0.f;      // in units of log 2: the decay is one exp2
   }
   const float skip = a.skip[c];
   __syncthreads();
   float steps = 0.f;
-  for (int tt = 0; tt < len; ++tt) {
-    const float d = Ds[tt * 64 + mine];
-    const float u = to_float(Us[tt * 64 + mine]);
-    const float du = d * u;
-    steps += d;
-    float b[KPT];
-    lds_row<KPT>(BCs + tt * 2 * NP + ng * KPT, b);
-    if (MODE == 1) {
+  if (MODE == 1) {
+    for (int tt = 0; tt < len; ++tt) {
+      const float d = Ds[tt * 64 + mine];
+      const float du = d * to_float(Us[tt * 64 + mine]);
+      steps += d;
+      float b[KPT];
+      lds_row<KPT>(BCs + tt * 2 * NP + ng * KPT, b);
 #pragma unroll
-      for (int k = 0; k < KPT; ++k) st[k] = fmaf(expf(d * ak[k]), st[k], du * b[k]);
-    } else {
-      float cv[KPT];
-      lds_row<KPT>(BCs + tt * 2 * NP + NP + ng * KPT, cv);
-      float y = 0.f;
+      for (int k = 0; k < KPT; ++k) st[k] = fmaf(__builtin_amdgcn_exp2f(d * ak[k]), st[k], du * b[k]);
+    }
+  } else {
+    // four tokens at a time: the four lanes of a channel exchange their shares so that lane ng ends with the whole sum
+    // of token ng, and every lane finishes and stores one token's output
+    for (int t0 = 0; t0 < len; t0 += 4) {
+      float part[4];
 #pragma unroll
-      for (int k = 0; k < KPT; ++k) {
-        st[k] = fmaf(expf(d * ak[k]), st[k], du * b[k]);
-        y = fmaf(st[k], cv[k], y);
+      for (int i = 0; i < 4; ++i) {
+        const int tt = min(t0 + i, len - 1);
+        const bool real = t0 + i < len;
+        const float d = real ? Ds[tt * 64 + mine] : 0.f;      // a step size of 0: the state stays as it is
+        const float du = d * to_float(Us[tt * 64 + mine]);
+        float b[KPT], cv[KPT];
+        lds_row<KPT>(BCs + tt * 2 * NP + ng * KPT, b);
+        lds_row<KPT>(BCs + tt * 2 * NP + NP + ng * KPT, cv);
+        float y = 0.f;
+#pragma unroll
+        for (int k = 0; k < KPT; ++k) {
+          st[k] = fmaf(__builtin_amdgcn_exp2f(d * ak[k]), st[k], du * b[k]);
+          y = fmaf(st[k], cv[k], y);
+        }
+        part[i] = y;
       }
-      y += __shfl_xor(y, 1, 64);
-      y += __shfl_xor(y, 2, 64);
-      if (ng == 0 && live)
-        ((T*)a.out)[size_t(q0 + tt) * a.inner + c] = from_float<T>(fmaf(skip, u, y) * silu_of(to_float(Zs[tt * 64 + mine])));
+      float two[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const float keep = (ng & 2) ? part[i + 2] : part[i], give = (ng & 2) ? part[i] : part[i + 2];
+        two[i] = keep + __shfl_xor(give, 2, 64);
+      }
+      const float keep = (ng & 1) ? two[1] : two[0], give = (ng & 1) ? two[0] : two[1];
+      const float y = keep + __shfl_xor(give, 1, 64);
+      const int tt = t0 + ng;
+      if (tt < len && live)
+        ((T*)a.out)[size_t(q0 + tt) * a.inner + c] =
+            from_float<T>(fmaf(skip, to_float(Us[tt * 64 + mine]), y) * silu_of(to_float(Zs[tt * 64 + mine])));
     }
   }
   if (MODE == 2 || !live) return;
@@ -771,6 +859,20 @@ extern "C" int sp_scale_rows(void* stream, int dtype, const void* x, const float
   return check_launch("sp_scale_rows");
 }
 
+// A kernel that asks for more than the 64 KB of LDS it gets unasked is told so once.
+template <auto Kernel>
+static bool more_lds(size_t bytes) {
+  static bool raised = false;      // one per kernel
+  if (bytes <= 64 * 1024 || raised) return true;
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+  if (e != hipSuccess) {
+    set_error("scan: cannot raise the LDS limit: %s", hipGetErrorString(e));
+    return false;
+  }
+  raised = true;
+  return true;
+}
+
 // Portions of more than kScanLong tokens are walked in chunks of kScanChunk.
 constexpr int kScanLong = 128;
 
@@ -803,7 +905,7 @@ extern "C" int sp_ssd_scan(void* stream, int dtype, const void* proj, long long 
              "sp_ssd_scan: null operand");
   if (T == 0 || n_seqs == 0) return 0;
   SsdArgs a = {proj, proj_stride, z_off, dt_off, xbc, xbc_stride, heads, vdim, state_size, groups, dt_bias, a_log, skip,
-               q_start, q_len, state_slots, state, out, 0, 1, nullptr, nullptr};
+               q_start, q_len, state_slots, state, out, 0, 1, nullptr, nullptr, 0};
   hipStream_t s = (hipStream_t)stream;
 #define SP_SSD_MODE(KPT, MODE)                                                       \
   do {                                                                               \
@@ -831,12 +933,21 @@ extern "C" int sp_ssd_scan(void* stream, int dtype, const void* proj, long long 
   // heads of whole 32s of values whose chunk fits 64 KB of LDS: the kernels that bring a chunk into LDS first
   const int kpt = state_size <= 32 ? 4 : state_size <= 64 ? 8 : state_size <= 128 ? 16 : 32;
   const size_t element = dtype == kF32 ? 4 : 2;
-  const size_t lds = 2 * kScanChunk * sizeof(float) + 2 * size_t(kScanChunk) * (8 * kpt + 32) * element;
-  const bool staged = vdim % 32 == 0 && lds <= 64 * 1024;
-#define SP_SSD_CHUNK_MODE(KPT, MODE)                                                    \
-  do {                                                                                  \
-    if (dtype == kF32) ssd_chunk_kernel<float, KPT, MODE><<<grid, 256, lds, s>>>(a);    \
-    else ssd_chunk_kernel<bf16_t, KPT, MODE><<<grid, 256, lds, s>>>(a);                 \
+  // MODE 1 holds B alone and the block's columns of u; MODE 2 also C and z
+  const size_t lds1 = size_t(kScanChunk) * ((2 + 8 * kpt) * sizeof(float) + 32 * element);
+  const size_t lds2 = size_t(kScanChunk) * (2 * sizeof(float) + (16 * kpt + 64) * element);
+  const bool staged = vdim % 32 == 0 && lds1 <= 96 * 1024 && lds2 <= 96 * 1024;
+  a.by_column = staged;
+#define SP_SSD_CHUNK_MODE(KPT, MODE)                                                                       \
+  do {                                                                                                     \
+    const size_t lds = MODE == 1 ? lds1 : lds2;                                                            \
+    if (dtype == kF32) {                                                                                   \
+      if (!more_lds<ssd_chunk_kernel<float, KPT, MODE>>(lds)) return 1;                                     \
+      ssd_chunk_kernel<float, KPT, MODE><<<grid, 256, lds, s>>>(a);                                        \
+    } else {                                                                                               \
+      if (!more_lds<ssd_chunk_kernel<bf16_t, KPT, MODE>>(lds)) return 1;                                    \
+      ssd_chunk_kernel<bf16_t, KPT, MODE><<<grid, 256, lds, s>>>(a);                                       \
+    }                                                                                                      \
   } while (0)
 #define SP_SSD_CHUNK(MODE)                          \
   do {                                              \

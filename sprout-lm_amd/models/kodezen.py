@@ -9,7 +9,8 @@ the mixer's input); the mixer's under `mix.` (mamba2: `in`, `conv`, `conv.b`, `d
 from __future__ import annotations
 
 from ..config.kodezen import KodezenConfig
-from .plan import LayerCall, LayerPlan, ModelPlan, PartPlan
+from ..parts.base import make_part
+from .plan import LayerCall, LayerPlan, ModelParts, ModelPlan, PartPlan
 
 # The design gives no position limit; the engine's bookkeeping wants one.
 MAX_POSITIONS = 1 << 22
@@ -57,21 +58,23 @@ def _layer(cfg: KodezenConfig, i: int) -> LayerPlan:
     return LayerPlan("pre_norm", parts)
 
 
+def _slots(layers: list) -> list:
+    """One cache slot per thing a layer's parts keep (pages, states, a convolution's last inputs), numbered in the order in
+    which the parts name them; what a part keeps is asked of the part itself."""
+    schedule, free = [], 0
+    for i, layer in enumerate(layers):
+        block = make_part("block", layer.block, **{name: part.make() for name, part in layer.parts.items()})
+        needs = ModelParts.cache_needs(block)
+        schedule.append(LayerCall(i, {key: free + n for n, key in enumerate(needs)} or None))
+        free += len(needs)
+    return schedule
+
+
 def build_kodezen(cfg: KodezenConfig) -> ModelPlan:
-    plan = ModelPlan(
+    layers = [_layer(cfg, i) for i in range(len(cfg.layers))]
+    return ModelPlan(
         architecture=cfg.architecture, config=cfg, hidden_size=cfg.width, vocab_size=cfg.vocab, max_positions=MAX_POSITIONS,
         eos_token_ids=(), embedding=PartPlan("embedding", "token_embedding", {"vocab": cfg.vocab, "hidden": cfg.width,
                                                                               "tensor": "embed", "scale": cfg.embedding_scale}),
-        layers=[_layer(cfg, i) for i in range(len(cfg.layers))], schedule=[],
-        final_norm=_norm(cfg, "final.norm"),
+        layers=layers, schedule=_slots(layers), final_norm=_norm(cfg, "final.norm"),
         head=PartPlan("head", "linear_head", {"vocab": cfg.vocab, "hidden": cfg.width, "tied": False, "tensor": "head"}))
-    # one cache slot per thing a layer's parts keep, in the order the parts name them
-    from .plan import ModelParts
-    free = 0
-    for i, layer in enumerate(plan.layers):
-        block_parts = {name: part.make() for name, part in layer.parts.items()}
-        from ..parts.base import make_part
-        needs = ModelParts.cache_needs(make_part("block", layer.block, **block_parts))
-        plan.schedule.append(LayerCall(i, {key: free + n for n, key in enumerate(needs)} or None))
-        free += len(needs)
-    return plan

@@ -28,6 +28,10 @@ def plain_side(folder: str, dtype: str):
         from tests.plain import bogilix_plain as B
         cfg, weights = B.load_folder(folder)
         return cfg, weights, B.forward
+    if name == "Kodezen":
+        from tests.plain import kodezen_plain as K
+        cfg, weights = K.load_folder(folder)
+        return cfg, weights, K.forward
     if name == "Megozen":
         from tests.plain import megozen_plain as M
         cfg, weights = M.load_folder(folder)
