@@ -103,7 +103,7 @@ def test_short_convolution_in_portions(dtype, channels, taps, bias, act, residua
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,vdim,state,groups,taps,parts", [(3, 10, 5, 1, 2, 3), (4, 32, 64, 1, 4, 2), (8, 16, 128, 4, 3, 4),
-                                                                (4, 6, 9, 2, 1, 1), (2, 64, 200, 2, 4, 1), (6, 32, 32, 2, 4, 2)])
+                                                                (4, 6, 9, 2, 1, 1), (2, 64, 200, 2, 4, 1), (6, 32, 48, 3, 4, 3)])
 def test_state_space_duality_alone_in_portions(dtype, heads, vdim, state, groups, taps, parts):
     from sprout_lm_amd.parts import make_part
     hidden, eps = 48, 1e-5
@@ -152,7 +152,7 @@ def test_a_slow_head_remembers_and_a_fast_head_forgets():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("inner,state,rank,taps", [(36, 5, 3, 4), (256, 16, 8, 4), (20, 1, 1, 1), (64, 40, 16, 2), (200, 130, 9, 3),
-                                                   (256, 24, 16, 3)])
+                                                   (192, 20, 12, 3)])
 def test_selective_scan_alone_in_portions(dtype, inner, state, rank, taps):
     from sprout_lm_amd.parts import make_part
     hidden = 48
@@ -186,7 +186,7 @@ def attention_sizes(heads, kv_heads, dim, scale, taps, rot_dims, base, mask):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,dim,taps,rot_dims,mask", [
     (6, 3, 12, 3, 8, (7, 2)), (3, 3, 20, 1, 0, None), (4, 1, 32, 4, 32, (24, 20)), (8, 4, 16, 2, 8, (64, 0)),
-    (6, 3, 16, 2, 16, (1, 0)), (4, 2, 128, 3, 64, (40, 4)), (2, 1, 48, 1, 24, (300, 1))])
+    (6, 3, 16, 2, 16, (1, 0)), (4, 2, 128, 3, 96, (48, 5)), (2, 1, 48, 1, 24, (300, 1))])
 def test_attention_alone_in_portions(dtype, heads, kv_heads, dim, taps, rot_dims, mask):
     hidden, eps, scale, base = 40, 1e-5, 0.7 / np.sqrt(dim), 200.0
     rng = np.random.default_rng(heads * 10 + dim)
@@ -207,7 +207,7 @@ def test_attention_keys_at_the_window_s_edges_and_kept_first_keys(dtype, page):
     """One flagged key whose score towers over its row and whose value is far from the rest: just inside the window, just
     outside, the last kept first key, the first one not kept, far away, at a page's first and last place; the reader in a
     portion of a prompt and decoded alone.  One key too many or too few moves the output by the size of a value."""
-    hidden, heads, kv_heads, dim, window, keep = 24, 4, 2, 16, 40, 4
+    hidden, heads, kv_heads, dim, window, keep = 24, 4, 2, 16, 36, 5
     scale, eps = 2.0, 1e-6
     part = attention_part(hidden, heads, kv_heads, dim, scale, 1, 8, 100.0, (window, keep), eps)
     rng = np.random.default_rng(5)
@@ -222,8 +222,8 @@ def test_attention_keys_at_the_window_s_edges_and_kept_first_keys(dtype, page):
     bind(part, w, dtype)
     m = attention_sizes(heads, kv_heads, dim, scale, 1, 8, 100.0, (window, keep))
     n = 260
-    for reader, key in ((200, 161), (200, 160), (200, 3), (200, 4), (200, 50), (231, 192), (231, 191), (96, 57), (95, 56),
-                        (259, 0), (41, 2), (43, 3), (39, 0), (44, 4)):
+    for reader, key in ((200, 165), (200, 164), (200, 4), (200, 5), (200, 50), (227, 192), (227, 191), (96, 61), (91, 56),
+                        (259, 0), (40, 4), (41, 5), (35, 0), (39, 3)):
         x = rounded(rng.standard_normal((n, hidden)) * 0.3, dtype)
         x[:, :2] = 0.0
         x[key, 0] = 4.0
@@ -232,7 +232,7 @@ def test_attention_keys_at_the_window_s_edges_and_kept_first_keys(dtype, page):
         seen = key <= reader and (reader - key < window or key < keep)
         lone = K.attention_mixer(w, "", m, np.where(np.arange(n)[:, None] == key, 0.0, x), np.arange(n), eps, store_of(dtype))
         assert (np.abs(want[reader] - lone[reader]).max() > 0.5) == seen, (reader, key)
-        for steps in ([(reader + 1,), (n,)], [(reader,), (1,), (n,)], [(37,), (reader - 37,), (1,), (1,), (n,)]):
+        for steps in ([(reader + 1,), (n,)], [(reader,), (1,), (n,)], [(33,), (reader - 33,), (1,), (1,), (n,)]):
             got = run_in_portions(part, specs_of(part), dtype, [x], steps, hidden, page=page)[0]
             close(got[reader], want[reader], dtype, f"reader {reader}, key {key}, steps {steps}", f32=3e-5, bf16=4e-2)
 
@@ -254,8 +254,8 @@ def test_dense_feed_forward_with_biases(dtype, hidden, inner, T):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden,inner,experts,top,T", [(100, 12, 5, 2, 9), (128, 64, 4, 1, 70), (64, 32, 8, 8, 33), (128, 96, 8, 1, 300),
-                                                        (256, 96, 8, 3, 1)])
+@pytest.mark.parametrize("hidden,inner,experts,top,T", [(100, 12, 5, 2, 9), (128, 64, 4, 1, 70), (64, 32, 8, 8, 33), (128, 80, 8, 1, 300),
+                                                        (256, 80, 6, 3, 1)])
 def test_routed_experts_weighted_on_their_input(dtype, hidden, inner, experts, top, T):
     """Sigmoid scores, the largest chosen, no renormalising, the weight on what the expert reads: silu is not linear, so a
     weight on the output instead shows."""
