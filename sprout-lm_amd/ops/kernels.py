@@ -1040,6 +1040,27 @@ def retention(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int
                                  T, n_seqs, int(max_q_len) if scratch is not None else 0, _ptr(scratch)))
 
 
+def gemm_from_residual(residual: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor, out: torch.Tensor,
+                       bias: torch.Tensor | None = None) -> bool:
+    """out (bfloat16 [T, N]) = (rmsnorm(residual) * norm_weight) . w^T (+ bias) in one kernel, for the few tokens of a decode
+    step: the norm is the product's prologue.  Returns False (and does nothing) where the kernel does not take the shape
+    or a norm kernel before the product would be faster; the caller then norms and multiplies in turn."""
+    N, K = w.shape
+    T = residual.shape[0]
+    if (w.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or tuple(out.shape) != (T, N) or T > 64
+            or not fused_supported(0, T, N, K, norm=True) or not fused_norm_pays(T, N, K)):
+        return False
+    _gpu(w, "weight"); _gpu(out, "output")
+    xp, rp, nd, npt, _ = _activations(None, residual, norm_weight, K, "gemm_from_residual")
+    if bias is not None:
+        _gpu(bias, "bias")
+        if bias.numel() != N:
+            raise KernelError(f"gemm_from_residual: bias has {bias.numel()} values for {N} columns")
+    check(library().sp_gemm_decode(_stream(), xp, rp, nd, npt, float(eps), w.data_ptr(), _code(bias, "bias") if bias is not None else 0,
+                                   _ptr(bias), STORE, out.data_ptr(), T, N, K))
+    return True
+
+
 def gate_up_silu(w: torch.Tensor, out: torch.Tensor, x=None, residual=None, norm_weight=None, eps: float = 0.0,
                  activation: str = "silu", limit: float = 0.0, row_gate=None, row_gate_column: int = 0) -> None:
     """out = act(a . w[:I]^T, a . w[I:]^T) for activations a as in `qkv_rope_cache`, times sigmoid(row_gate[t, column])

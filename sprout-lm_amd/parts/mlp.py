@@ -128,6 +128,19 @@ class DenseMLP(FeedForward):
         self.b_down = tensors[down + self.bias] if self.bias is not None else None
         self.w = {}
 
+    def forward_from_residual(self, ctx, norm, residual) -> bool:
+        """A decode step's few tokens: the norm as the prologue of the up product, a launch less."""
+        fold = norm.fold()
+        if fold is None or fold.kind != "rms" or ctx.act_dtype != torch.bfloat16:
+            return False
+        T = residual.shape[0]
+        act = ctx.buffer("mlp_inner", (T, self.inner), ctx.act_dtype)
+        if not ops.gemm_from_residual(residual, fold.weight, fold.eps, self.w_up, act, bias=self.b_up):
+            return False
+        ops.activation(act, self.activation)
+        ops.gemm(act, self.w_down, residual, bias=self.b_down, accumulate=True)
+        return True
+
     def forward(self, ctx, h, residual):
         T = h.shape[0]
         act = ctx.buffer("mlp_inner", (T, self.inner), ctx.act_dtype)

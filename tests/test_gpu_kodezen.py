@@ -251,6 +251,16 @@ def test_dense_feed_forward_with_biases(dtype, hidden, inner, T):
     residual = torch.zeros(T, hidden, device=DEV)
     part.forward(ctx, dev(x, dtype), residual)
     close(residual.cpu().numpy(), K.dense_ff(w, "", x, store_of(dtype)), dtype, "dense feed-forward")
+    # from the residual stream, the norm folded into the first product where a kernel does that (few tokens, bfloat16)
+    norm = make_part("norm", "rmsnorm", size=hidden, eps=1e-5, tensor="n", one_plus=True)
+    nw = rounded(rng.normal(0, 0.1, hidden), dtype)
+    bind(norm, {"n": nw}, dtype)
+    stream = (rng.standard_normal((T, hidden)) * 3.0).astype(np.float32)
+    residual = dev(stream)
+    if part.forward_from_residual(ctx, norm, residual):
+        want = stream + K.dense_ff(w, "", store_of(dtype)(K.one_plus_norm(stream, nw, 1e-5)), store_of(dtype))
+        close(residual.cpu().numpy(), want, dtype, "dense feed-forward from the residual")
+        print(f"norm folded into the product: hidden {hidden}, inner {inner}, {T} tokens")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
