@@ -435,7 +435,11 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   const StepRule rule = step_rule(st, scale2);
 
   const int32_t* table = block_tables + size_t(seq) * max_blocks;
-  const int first_page = k_lo >> page_shift, n_pages = (k_hi >> page_shift) - first_page + 1;
+  // the stage of the first key the tile's rows see; kept first keys that reach into it are loaded with it (the page
+  // numbers in LDS then start at the stage's first page), those before it in stages of their own (below)
+  const int lo_stage = (k_lo / kStageKeys) * kStageKeys;
+  const int table_lo = st.keep > lo_stage ? lo_stage : k_lo;
+  const int first_page = table_lo >> page_shift, n_pages = (k_hi >> page_shift) - first_page + 1;
   const bool table_in_lds = n_pages <= kMaxTableLds;
   if (table_in_lds)
     for (int i = threadIdx.x; i < n_pages; i += THREADS) s_table[i] = table[first_page + i];
@@ -494,13 +498,17 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   constexpr bool ROWWISE = KCHUNKS % THREADS == 0 && (HD / 8) % (PER_K > 0 ? PER_K : 1) == 0 && THREADS % 16 == 0;
   constexpr int KT = ROWWISE ? (HD / 8) / PER_K : 1, VD = THREADS / 16;
   const int kr = threadIdx.x / KT, kc = threadIdx.x % KT, vc = threadIdx.x % 16, vd = threadIdx.x / 16;
+  // the keys a fetch may take: k_lo .. k_hi; from the stage's own first key where kept first keys reach into it (what
+  // lies between them and k_lo is masked by position, and a page number that is none is clamped); 0 .. the last kept key
+  // for a stage of kept keys alone
+  int f_lo = st.keep > lo_stage ? lo_stage : k_lo, f_hi = k_hi;
   auto fetch_from = [&](uint4 (&stage)[PER_THREAD], int key0, auto in_lds) __attribute__((always_inline)) {
-    const bool interior = key0 >= k_lo && key0 + kStageKeys - 1 <= k_hi;   // no key of the stage needs clamping
+    const bool interior = key0 >= f_lo && key0 + kStageKeys - 1 <= f_hi;   // no key of the stage needs clamping
     if constexpr (ROWWISE) {
       int key = key0 + kr, kb = key0 + 8 * vc;
       if (!interior) {
-        key = min(max(key, k_lo), k_hi);
-        kb = min(max(kb, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
+        key = min(max(key, f_lo), f_hi);
+        kb = min(max(kb, (f_lo >> 3) << 3), (f_hi >> 3) << 3);
       }
       const uint16_t* krow = kbase + (((size_t(page_at(key, in_lds)) * heads) << page_shift) + (key & page_mask)) * HD + 8 * kc;
       const uint16_t* vcol = vbase + ((size_t(page_at(kb, in_lds)) * heads * HD + size_t(vd)) << page_shift) + (kb & page_mask);
@@ -516,12 +524,12 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
       if (i < KCHUNKS) {                       // keys: row r of the stage, dims 8 c .. 8 c + 7
         const int r = i / (HD / 8), c = i % (HD / 8);
         int key = key0 + r;
-        if (!interior) key = min(max(key, k_lo), k_hi);
+        if (!interior) key = min(max(key, f_lo), f_hi);
         stage[u] = ldg128(kbase + (((size_t(page_at(key, in_lds)) * heads) << page_shift) + (key & page_mask)) * HD + 8 * c);
       } else if (i < CHUNKS) {                 // values: dim d, keys 8 c .. 8 c + 7 of the stage
         const int j = i - KCHUNKS, d = j / (kStageKeys / 8), c = j % (kStageKeys / 8);
         int kb = key0 + 8 * c;
-        if (!interior) kb = min(max(kb, (k_lo >> 3) << 3), (k_hi >> 3) << 3);
+        if (!interior) kb = min(max(kb, (f_lo >> 3) << 3), (f_hi >> 3) << 3);
         stage[u] = ldg128(vbase + ((size_t(page_at(kb, in_lds)) * heads * HD + size_t(d)) << page_shift) + (kb & page_mask));
       }
     }
@@ -559,7 +567,7 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
     for (int sub = 0; sub < WAVE_KEYS / 32; ++sub) {
       const int skey = WAVE_KEYS * wave + 32 * sub;
       const int wkey = key0 + skey;
-      if (has_head && wkey <= k_hi && wkey + 32 > k_lo) {
+      if (has_head && wkey <= k_hi && (wkey + 32 > k_lo || wkey < st.keep)) {
         KVStep<DT> r;
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
@@ -583,6 +591,20 @@ __global__ __launch_bounds__(64 * WPT * HPB) void attention_prefill_staged_kerne
   };
   uint4 stage[PER_THREAD];
   __syncthreads();   // the page numbers are in LDS
+  if (st.keep > 0 && split == 0) {
+    // the stages of kept first keys that lie wholly before the window's first stage: the block of the first split walks
+    // them first, their page numbers read from memory (the numbers in LDS start later)
+    const int window_lo = f_lo;
+    f_lo = 0;
+    f_hi = min(st.keep - 1, k_hi);
+    for (int key0 = 0; key0 < min(st.keep, lo_stage); key0 += kStageKeys) {
+      fetch_from(stage, key0, std::false_type{});
+      to_lds(stage);
+      use_stage(key0);
+    }
+    f_lo = window_lo;
+    f_hi = k_hi;
+  }
   if (AHEAD && range_lo <= range_hi) fetch(stage, range_lo);
   for (int key0 = range_lo; key0 <= range_hi; key0 += kStageKeys) {
     if (!AHEAD) fetch(stage, key0);
@@ -1082,7 +1104,7 @@ static int launch_mfma(hipStream_t s, const void* q, int q_stride, const void* k
   // the workspace holds the decode partials first, then the prefill partials
   float* prefill_ws = workspace ? workspace + attention_decode_workspace_floats(n_decode, nq, HD, max_decode_ctx) : nullptr;
   if (n_tiles > 0) {
-    if (staged_prefill(page_size) && st.keep == 0) {      // (kept first keys: the walk of the one-wave kernel knows them)
+    if (staged_prefill(page_size)) {
       int page_shift = 0;
       while ((1 << page_shift) < page_size) ++page_shift;
       const int splits = attention_prefill_splits(n_tiles, nq, nkv, HD, page_size, max_tile_ctx);
