@@ -186,7 +186,8 @@ def attention_sizes(heads, kv_heads, dim, scale, taps, rot_dims, base, mask):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,dim,taps,rot_dims,mask", [
     (6, 3, 12, 3, 8, (7, 2)), (3, 3, 20, 1, 0, None), (4, 1, 32, 4, 32, (24, 20)), (8, 4, 16, 2, 8, (64, 0)),
-    (6, 3, 16, 2, 16, (1, 0)), (4, 2, 128, 3, 96, (48, 5)), (2, 1, 48, 1, 24, (300, 1))])
+    (6, 3, 16, 2, 16, (1, 0)), (4, 2, 128, 3, 96, (48, 5)), (2, 1, 48, 1, 24, (300, 1)), (4, 2, 32, 2, 16, (20, 150)),
+    (2, 1, 64, 1, 0, (10, 300))])
 def test_attention_alone_in_portions(dtype, heads, kv_heads, dim, taps, rot_dims, mask):
     hidden, eps, scale, base = 40, 1e-5, 0.7 / np.sqrt(dim), 200.0
     rng = np.random.default_rng(heads * 10 + dim)
