@@ -217,16 +217,18 @@ struct SsdArgs {
 //   MODE 2  every chunk again, from the state it starts from, with the outputs.
 // MODE 0 walks a request's tokens in one go (short portions, single tokens).  blockIdx.y: the request (MODE 0), or
 // request * chunks_per_request + chunk.
-template <typename T, int KPT, int MODE>
+// CP: the neighbouring columns a lane holds (2 where a head's values are an even number: a row's numbers are then read
+// and written eight bytes a lane, 64 bytes a run, and B and C are fetched once for both).
+template <typename T, int KPT, int MODE, int CP>
 __global__ __launch_bounds__(256) void ssd_scan_kernel(SsdArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int rg = lane & 7, pc = lane >> 3;
   const int inner = a.heads * a.vdim, N = a.state_size;
   const int s = MODE == 0 ? blockIdx.y : blockIdx.y / a.chunks;
   const int ci = MODE == 0 ? 0 : blockIdx.y % a.chunks;
-  int col = blockIdx.x * 32 + wave * 8 + pc;
+  int col = (blockIdx.x * 32 + wave * 8 + pc) * CP;
   const bool live = col < inner;
-  if (!live) col = inner - 1;      // the lane stays for its neighbours' sums and stores nothing
+  if (!live) col = inner - CP;      // the lane stays for its neighbours' sums and stores nothing
   const int n = col / a.vdim, p = col % a.vdim, g = n / (a.heads / a.groups);
   int q0 = a.q_start[s], L = a.q_len[s];
   if (MODE != 0) {
@@ -234,14 +236,24 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(SsdArgs a) {
     L = min(a.chunk, L - ci * a.chunk);
   }
   if (L <= 0) return;
-  // the state rows of this column: the request's own (MODE 0), or the chunk's place in the scratch
+  // the state rows of these columns: the request's own (MODE 0), or the chunk's place in the scratch
   float* S = MODE == 0 ? a.state + ((size_t(a.state_slots[s]) * a.heads + n) * N) * a.vdim + p
                        : a.scratch + ((size_t(blockIdx.y) * a.heads + n) * N) * a.vdim + p;
-  float st[KPT];
+  float st[KPT][CP];
 #pragma unroll
   for (int k = 0; k < KPT; ++k) {
     const int r = rg + 8 * k;
-    st[k] = (MODE != 1 && r < N) ? S[size_t(r) * a.vdim] : 0.f;
+#pragma unroll
+    for (int j = 0; j < CP; ++j) st[k][j] = 0.f;
+    if (MODE != 1 && r < N) {
+      if (CP == 2) {
+        const float2 v = *reinterpret_cast<const float2*>(S + size_t(r) * a.vdim);
+        st[k][0] = v.x;
+        st[k][CP - 1] = v.y;
+      } else {
+        st[k][0] = S[size_t(r) * a.vdim];
+      }
+    }
   }
   const float rate = expf(a.a_log[n]), bias = a.dt_bias[n], skip = a.skip[n];
   const T* proj = (const T*)a.proj;
@@ -253,23 +265,39 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(SsdArgs a) {
     const T* xr = xbc + size_t(t) * a.xbc_stride;
     const float d = softplus_of(to_float(pr[a.dt_off + n]) + bias);
     const float decay = expf(-rate * d);
-    const float u = to_float(xr[col]);
-    const float du = d * u;
+    float u[CP], du[CP], y[CP];
+#pragma unroll
+    for (int j = 0; j < CP; ++j) {
+      u[j] = to_float(xr[col + j]);
+      du[j] = d * u[j];
+      y[j] = 0.f;
+    }
     steps += d;
-    float y = 0.f;
 #pragma unroll
     for (int k = 0; k < KPT; ++k) {
       const int r = rg + 8 * k;
       if (r < N) {
-        st[k] = fmaf(decay, st[k], du * to_float(xr[b_off + r]));
-        if (MODE != 1) y = fmaf(st[k], to_float(xr[c_off + r]), y);
+        const float b = to_float(xr[b_off + r]);
+        const float c = MODE != 1 ? to_float(xr[c_off + r]) : 0.f;
+#pragma unroll
+        for (int j = 0; j < CP; ++j) {
+          st[k][j] = fmaf(decay, st[k][j], du[j] * b);
+          if (MODE != 1) y[j] = fmaf(st[k][j], c, y[j]);
+        }
       }
     }
     if (MODE != 1) {
-      y += __shfl_xor(y, 1, 64);
-      y += __shfl_xor(y, 2, 64);
-      y += __shfl_xor(y, 4, 64);
-      if (rg == 0 && live) a.out[size_t(t) * inner + col] = fmaf(skip, u, y) * silu_of(to_float(pr[a.z_off + col]));
+#pragma unroll
+      for (int j = 0; j < CP; ++j) {
+        y[j] += __shfl_xor(y[j], 1, 64);
+        y[j] += __shfl_xor(y[j], 2, 64);
+        y[j] += __shfl_xor(y[j], 4, 64);
+      }
+      if (rg == 0 && live) {
+#pragma unroll
+        for (int j = 0; j < CP; ++j)
+          a.out[size_t(t) * inner + col + j] = fmaf(skip, u[j], y[j]) * silu_of(to_float(pr[a.z_off + col + j]));
+      }
     }
   }
   if (MODE == 2) return;
@@ -277,7 +305,10 @@ __global__ __launch_bounds__(256) void ssd_scan_kernel(SsdArgs a) {
 #pragma unroll
     for (int k = 0; k < KPT; ++k) {
       const int r = rg + 8 * k;
-      if (r < N) S[size_t(r) * a.vdim] = st[k];
+      if (r < N) {
+        if (CP == 2) *reinterpret_cast<float2*>(S + size_t(r) * a.vdim) = make_float2(st[k][0], st[k][CP - 1]);
+        else S[size_t(r) * a.vdim] = st[k][0];
+      }
     }
     if (MODE == 1 && p == 0 && rg == 0) a.step_sums[size_t(blockIdx.y) * a.heads + n] = steps;
   }
@@ -933,10 +964,15 @@ extern "C" int sp_ssd_scan(void* stream, int dtype, const void* proj, long long 
   SsdArgs a = {proj, proj_stride, z_off, dt_off, xbc, xbc_stride, heads, vdim, state_size, groups, dt_bias, a_log, skip,
                q_start, q_len, state_slots, state, out, 0, 1, nullptr, nullptr, 0};
   hipStream_t s = (hipStream_t)stream;
-#define SP_SSD_MODE(KPT, MODE)                                                       \
-  do {                                                                               \
-    if (dtype == kF32) ssd_scan_kernel<float, KPT, MODE><<<grid, 256, 0, s>>>(a);    \
-    else ssd_scan_kernel<bf16_t, KPT, MODE><<<grid, 256, 0, s>>>(a);                 \
+  // two neighbouring columns a lane where a head's values are an even number and rows start at eight bytes
+  const bool pairs = vdim % 2 == 0 && (reinterpret_cast<uintptr_t>(state) & 7) == 0 && (!scratch || (reinterpret_cast<uintptr_t>(scratch) & 7) == 0);
+  const int columns = pairs ? 64 : 32;
+#define SP_SSD_MODE(KPT, MODE)                                                                    \
+  do {                                                                                            \
+    if (dtype == kF32 && pairs) ssd_scan_kernel<float, KPT, MODE, 2><<<grid, 256, 0, s>>>(a);     \
+    else if (dtype == kF32) ssd_scan_kernel<float, KPT, MODE, 1><<<grid, 256, 0, s>>>(a);         \
+    else if (pairs) ssd_scan_kernel<bf16_t, KPT, MODE, 2><<<grid, 256, 0, s>>>(a);                \
+    else ssd_scan_kernel<bf16_t, KPT, MODE, 1><<<grid, 256, 0, s>>>(a);                           \
   } while (0)
 #define SP_SSD(MODE)                                  \
   do {                                                \
@@ -947,7 +983,7 @@ extern "C" int sp_ssd_scan(void* stream, int dtype, const void* proj, long long 
   } while (0)
   const long long need = sp_ssd_scan_scratch_floats(heads, vdim, state_size, n_seqs, max_q_len);
   if (need == 0 || !scratch) {
-    const dim3 grid((inner + 31) / 32, n_seqs);
+    const dim3 grid((inner + columns - 1) / columns, n_seqs);
     SP_SSD(0);
     return check_launch("sp_ssd_scan");
   }
@@ -982,13 +1018,20 @@ extern "C" int sp_ssd_scan(void* stream, int dtype, const void* proj, long long 
     else if (kpt == 16) SP_SSD_CHUNK_MODE(16, MODE);\
     else SP_SSD_CHUNK_MODE(32, MODE);               \
   } while (0)
+  const dim3 staged_grid = grid;
   if (staged) SP_SSD_CHUNK(1);
-  else SP_SSD(1);
+  else {
+    const dim3 grid((inner + columns - 1) / columns, staged_grid.y);
+    SP_SSD(1);
+  }
   if (check_launch("sp_ssd_scan (chunks)")) return 1;
   ssd_carry_kernel<<<dim3((size_t(inner) * state_size + 255) / 256, n_seqs), 256, 0, s>>>(a);
   if (check_launch("sp_ssd_scan (carry)")) return 1;
   if (staged) SP_SSD_CHUNK(2);
-  else SP_SSD(2);
+  else {
+    const dim3 grid((inner + columns - 1) / columns, staged_grid.y);
+    SP_SSD(2);
+  }
 #undef SP_SSD_CHUNK
 #undef SP_SSD_CHUNK_MODE
 #undef SP_SSD
