@@ -103,7 +103,7 @@ def test_short_convolution_in_portions(dtype, channels, taps, bias, act, residua
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,vdim,state,groups,taps,parts", [(3, 10, 5, 1, 2, 3), (4, 32, 64, 1, 4, 2), (8, 16, 128, 4, 3, 4),
-                                                                (4, 6, 9, 2, 1, 1), (2, 64, 200, 2, 4, 1), (6, 32, 48, 3, 4, 3)])
+                                                                (4, 6, 9, 2, 1, 1), (2, 64, 200, 2, 4, 1), (6, 32, 48, 3, 4, 3), (2, 32, 128, 1, 2, 1)])
 def test_state_space_duality_alone_in_portions(dtype, heads, vdim, state, groups, taps, parts):
     from sprout_lm_amd.parts import make_part
     hidden, eps = 48, 1e-5
